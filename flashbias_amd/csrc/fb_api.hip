@@ -1,0 +1,239 @@
+// C ABI of the library (declared in include/flashbias.h): argument checks that run without
+// a GPU, translation of fb_params into kernel argument blocks, dispatch to the instantiation
+// that covers (dtype, head dim, rank).
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+
+#include "flashbias.h"
+#include "fb_kernels.h"
+
+namespace fb {
+#define FB_DECL(sfx)                                                          \
+    hipError_t launch_fwd_##sfx(const FwdArgs &a, hipStream_t stream);        \
+    hipError_t launch_bwd_main_##sfx(const BwdArgs &a, hipStream_t stream);
+FB_DECL(bf16_1) FB_DECL(bf16_2) FB_DECL(bf16_4) FB_DECL(bf16_8)
+FB_DECL(f16_1) FB_DECL(f16_2) FB_DECL(f16_4) FB_DECL(f16_8)
+#undef FB_DECL
+
+hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream) {
+    switch (nkd_of(a.d)) {
+    case 1: return bf16 ? launch_fwd_bf16_1(a, stream) : launch_fwd_f16_1(a, stream);
+    case 2: return bf16 ? launch_fwd_bf16_2(a, stream) : launch_fwd_f16_2(a, stream);
+    case 4: return bf16 ? launch_fwd_bf16_4(a, stream) : launch_fwd_f16_4(a, stream);
+    default: return bf16 ? launch_fwd_bf16_8(a, stream) : launch_fwd_f16_8(a, stream);
+    }
+}
+
+hipError_t launch_bwd_main(const BwdArgs &a, bool bf16, hipStream_t stream) {
+    switch (nkd_of(a.d)) {
+    case 1: return bf16 ? launch_bwd_main_bf16_1(a, stream) : launch_bwd_main_f16_1(a, stream);
+    case 2: return bf16 ? launch_bwd_main_bf16_2(a, stream) : launch_bwd_main_f16_2(a, stream);
+    case 4: return bf16 ? launch_bwd_main_bf16_4(a, stream) : launch_bwd_main_f16_4(a, stream);
+    default: return bf16 ? launch_bwd_main_bf16_8(a, stream) : launch_bwd_main_f16_8(a, stream);
+    }
+}
+} // namespace fb
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char *fmt, const char *what = "") {
+    std::snprintf(g_err, sizeof(g_err), fmt, what);
+    return code;
+}
+
+bool vec_ok(const fb_tensor &t) {
+    return (reinterpret_cast<uintptr_t>(t.ptr) % 16 == 0) && t.stride_b % 8 == 0 && t.stride_h % 8 == 0 &&
+           t.stride_s % 8 == 0;
+}
+
+fb::Tensor dev(const fb_tensor &t) {
+    fb::Tensor o;
+    o.ptr = static_cast<const uint16_t *>(t.ptr);
+    o.sb = t.stride_b;
+    o.sh = t.stride_h;
+    o.ss = t.stride_s;
+    o.vec_ok = vec_ok(t) ? 1 : 0;
+    return o;
+}
+
+fb::MaskDesc dev_mask(const fb_params *p) {
+    fb::MaskDesc m;
+    m.ptr = p->mask_type ? p->mask.ptr : nullptr;
+    m.sb = p->mask.stride_b;
+    m.sh = p->mask.stride_h;
+    m.sm = p->mask_type == FB_MASK_MATRIX ? p->mask.stride_s : 0;
+    m.type = p->mask_type;
+    m.is_f32 = p->mask_dtype == FB_F32;
+    return m;
+}
+
+// input: may broadcast over batch / head (stride 0), never negative strides
+int check_in(const fb_tensor &t, int channels, const char *name) {
+    if (!t.ptr) return fail(FB_ERR_NULL, "%s: null pointer", name);
+    if (t.stride_b < 0 || t.stride_h < 0 || t.stride_s < 0) return fail(FB_ERR_STRIDE, "%s: negative stride", name);
+    (void)channels;
+    return FB_OK;
+}
+
+// output: rows must not alias each other
+int check_out(const fb_tensor &t, int channels, int B, int H, int L, const char *name) {
+    if (!t.ptr) return fail(FB_ERR_NULL, "%s: null pointer", name);
+    if (t.stride_b < 0 || t.stride_h < 0 || t.stride_s < 0) return fail(FB_ERR_STRIDE, "%s: negative stride", name);
+    if ((L > 1 && t.stride_s < channels) || (B > 1 && t.stride_b == 0) || (H > 1 && t.stride_h == 0))
+        return fail(FB_ERR_STRIDE, "%s: output rows alias (zero or too small stride)", name);
+    return FB_OK;
+}
+
+uint64_t lq_pad_of(const fb_params *p) { return (static_cast<uint64_t>(p->Lq) + 31) / 32 * 32; }
+
+fb::FwdArgs fwd_args(const fb_params *p) {
+    fb::FwdArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.q = dev(p->q);
+    a.k = dev(p->k);
+    a.v = dev(p->v);
+    a.o = dev(p->o);
+    if (p->r > 0) {
+        a.qb = dev(p->q_bias);
+        a.kb = dev(p->k_bias);
+    }
+    a.mask = dev_mask(p);
+    a.lse = p->lse;
+    a.B = p->B; a.H = p->H; a.Lq = p->Lq; a.Lk = p->Lk; a.d = p->d; a.r = p->r;
+    a.causal = p->causal ? 1 : 0;
+    a.scale = p->scale;
+    return a;
+}
+
+fb::BwdArgs bwd_args(const fb_params *p) {
+    fb::BwdArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.q = dev(p->q);
+    a.k = dev(p->k);
+    a.v = dev(p->v);
+    a.o = dev(p->o);
+    a.dout = dev(p->dout);
+    a.dq = dev(p->dq);
+    a.dk = dev(p->dk);
+    a.dv = dev(p->dv);
+    if (p->r > 0) {
+        a.qb = dev(p->q_bias);
+        a.kb = dev(p->k_bias);
+        a.dqb = dev(p->dq_bias);
+        a.dkb = dev(p->dk_bias);
+    }
+    a.mask = dev_mask(p);
+    a.lse = p->lse;
+    a.delta = p->delta;
+    a.dq_acc = static_cast<float *>(p->workspace);
+    a.lq_pad = static_cast<int64_t>(lq_pad_of(p));
+    a.dq_rows = p->d + p->r;
+    a.r_row0 = p->d;
+    a.B = p->B; a.H = p->H; a.Lq = p->Lq; a.Lk = p->Lk; a.d = p->d; a.r = p->r;
+    a.causal = p->causal ? 1 : 0;
+    a.scale = p->scale;
+    return a;
+}
+
+int launched(hipError_t e, const char *what) {
+    if (e == hipSuccess) return FB_OK;
+    std::snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
+    return FB_ERR_LAUNCH;
+}
+
+} // namespace
+
+extern "C" {
+
+int fb_version(void) { return FB_VERSION; }
+
+const char *fb_last_error(void) { return g_err; }
+
+uint64_t fb_bwd_workspace_bytes(const fb_params *p) {
+    if (!p || p->B <= 0 || p->H <= 0 || p->Lq <= 0 || p->d <= 0 || p->r < 0) return 0;
+    return static_cast<uint64_t>(p->B) * p->H * (p->d + p->r) * lq_pad_of(p) * sizeof(float);
+}
+
+int fb_check(const fb_params *p, int pass) {
+    g_err[0] = 0;
+    if (!p) return fail(FB_ERR_NULL, "params: null pointer");
+    if (p->size != sizeof(fb_params)) return fail(FB_ERR_ABI, "fb_params.size does not match this library");
+    if (p->dtype != FB_F16 && p->dtype != FB_BF16) return fail(FB_ERR_DTYPE, "only fp16 and bf16 are supported");
+    if (p->B <= 0 || p->H <= 0 || p->Lq <= 0 || p->Lk <= 0) return fail(FB_ERR_SHAPE, "B, H, Lq, Lk must be positive");
+    if (p->d <= 0 || p->d > FB_MAX_HEADDIM) return fail(FB_ERR_SHAPE, "head dim must be in 1..128");
+    if (p->r < 0 || p->r > FB_MAX_RANK) return fail(FB_ERR_SHAPE, "bias rank must be in 0..128");
+    if (!std::isfinite(p->scale) || p->scale == 0.f) return fail(FB_ERR_SCALE, "softmax scale must be finite and non-zero");
+    int rc;
+    if ((rc = check_in(p->q, p->d, "q"))) return rc;
+    if ((rc = check_in(p->k, p->d, "k"))) return rc;
+    if ((rc = check_in(p->v, p->d, "v"))) return rc;
+    if (p->r > 0) {
+        if ((rc = check_in(p->q_bias, p->r, "q_bias"))) return rc;
+        if ((rc = check_in(p->k_bias, p->r, "k_bias"))) return rc;
+    }
+    if (p->mask_type != FB_MASK_NONE) {
+        if (p->mask_type != FB_MASK_VECTOR && p->mask_type != FB_MASK_MATRIX)
+            return fail(FB_ERR_MASK, "mask_type must be none, vector or matrix");
+        if (p->mask_dtype != p->dtype && p->mask_dtype != FB_F32)
+            return fail(FB_ERR_MASK, "mask must have the input dtype or fp32");
+        if (!p->mask.ptr) return fail(FB_ERR_NULL, "%s: null pointer", "mask");
+        if (p->mask.stride_b < 0 || p->mask.stride_h < 0 || p->mask.stride_s < 0)
+            return fail(FB_ERR_STRIDE, "%s: negative stride", "mask");
+    }
+    if (!p->lse) return fail(FB_ERR_NULL, "%s: null pointer", "lse");
+    if (pass == 0) return check_out(p->o, p->d, p->B, p->H, p->Lq, "o");
+    if ((rc = check_in(p->o, p->d, "o"))) return rc;
+    if ((rc = check_in(p->dout, p->d, "dout"))) return rc;
+    if ((rc = check_out(p->dq, p->d, p->B, p->H, p->Lq, "dq"))) return rc;
+    if ((rc = check_out(p->dk, p->d, p->B, p->H, p->Lk, "dk"))) return rc;
+    if ((rc = check_out(p->dv, p->d, p->B, p->H, p->Lk, "dv"))) return rc;
+    if (p->r > 0) {
+        if ((rc = check_out(p->dq_bias, p->r, p->B, p->H, p->Lq, "dq_bias"))) return rc;
+        if ((rc = check_out(p->dk_bias, p->r, p->B, p->H, p->Lk, "dk_bias"))) return rc;
+    }
+    if (!p->delta) return fail(FB_ERR_NULL, "%s: null pointer", "delta");
+    if (!p->workspace || p->workspace_bytes < fb_bwd_workspace_bytes(p))
+        return fail(FB_ERR_WORKSPACE, "workspace missing or smaller than fb_bwd_workspace_bytes()");
+    if (reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0)
+        return fail(FB_ERR_WORKSPACE, "workspace must be 16-byte aligned");
+    return FB_OK;
+}
+
+int fb_fwd(const fb_params *p, void *stream) {
+    const int rc = fb_check(p, 0);
+    if (rc) return rc;
+    return launched(fb::launch_fwd(fwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_fwd");
+}
+
+int fb_bwd_preprocess(const fb_params *p, void *stream) {
+    const int rc = fb_check(p, 1);
+    if (rc) return rc;
+    return launched(fb::launch_bwd_preprocess(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                    "fb_bwd_preprocess");
+}
+
+int fb_bwd_main(const fb_params *p, void *stream) {
+    const int rc = fb_check(p, 1);
+    if (rc) return rc;
+    return launched(fb::launch_bwd_main(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                    "fb_bwd_main");
+}
+
+int fb_bwd_finalize(const fb_params *p, void *stream) {
+    const int rc = fb_check(p, 1);
+    if (rc) return rc;
+    return launched(fb::launch_bwd_finalize(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                    "fb_bwd_finalize");
+}
+
+int fb_bwd(const fb_params *p, void *stream) {
+    int rc = fb_bwd_preprocess(p, stream);
+    if (rc) return rc;
+    if ((rc = fb_bwd_main(p, stream))) return rc;
+    return fb_bwd_finalize(p, stream);
+}
+
+} // extern "C"

@@ -1,0 +1,118 @@
+// Device-side building blocks shared by the forward and backward kernels (gfx950 only).
+//
+// MFMA tile used everywhere: v_mfma_f32_32x32x16_{bf16,f16}.  For a wave of 64 lanes with
+// g = lane / 32 and c = lane % 32:
+//   A operand (32 x 16): lane holds row c, eight consecutive k-slots of group g
+//   B operand (16 x 32): lane holds column c, eight consecutive k-slots of group g
+//   C / D    (32 x 32): lane holds column c, register v holds row 8*(v/4) + 4*g + v%4
+// Only the C layout is relied on; the pairing of k-slots between A and B is whatever the
+// hardware does, identical on both sides.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fb {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 f16x8_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct BF16 {
+    typedef uint16_t raw;
+    static __device__ __forceinline__ f32x16_t mfma(u32x4_t a, u32x4_t b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                       __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        bf16x2_t p;
+        p[0] = (__bf16)lo;
+        p[1] = (__bf16)hi;
+        return __builtin_bit_cast(uint32_t, p);
+    }
+    static __device__ __forceinline__ float to_float(uint16_t x) {
+        return __builtin_bit_cast(float, (uint32_t)x << 16);
+    }
+    static __device__ __forceinline__ uint16_t from_float(float x) {
+        return __builtin_bit_cast(uint16_t, (__bf16)x);
+    }
+    static constexpr uint16_t kOne = 0x3f80;
+};
+
+struct F16 {
+    typedef uint16_t raw;
+    static __device__ __forceinline__ f32x16_t mfma(u32x4_t a, u32x4_t b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                      __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+        f16x2_t p;
+        p[0] = (_Float16)lo;
+        p[1] = (_Float16)hi;
+        return __builtin_bit_cast(uint32_t, p);
+    }
+    static __device__ __forceinline__ float to_float(uint16_t x) {
+        return (float)__builtin_bit_cast(_Float16, x);
+    }
+    static __device__ __forceinline__ uint16_t from_float(float x) {
+        return __builtin_bit_cast(uint16_t, (_Float16)x);
+    }
+    static constexpr uint16_t kOne = 0x3c00;
+};
+
+// A (batch, seq, heads, channels) tensor as the kernels see it: 16-bit elements, channel
+// stride 1, everything else through element strides.
+struct Tensor {
+    const uint16_t *ptr;
+    int64_t sb, sh, ss;
+    int vec_ok; // base pointer and all strides are multiples of 16 bytes
+};
+
+struct MaskDesc {
+    const void *ptr;
+    int64_t sb, sh, sm;
+    int type;   // 0 none, 1 vector, 2 matrix
+    int is_f32; // else same 16-bit type as the inputs
+};
+
+// Eight consecutive channels [col0, col0 + 8) of one row; zero beyond ncols.
+__device__ __forceinline__ u32x4_t load_chunk(const uint16_t *row, int col0, int ncols, bool vec_ok) {
+    u32x4_t out = {0u, 0u, 0u, 0u};
+    if (col0 + 8 <= ncols && vec_ok) {
+        out = *reinterpret_cast<const u32x4_t *>(row + col0);
+    } else if (col0 < ncols) {
+        uint16_t e[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) e[i] = (col0 + i < ncols) ? row[col0 + i] : (uint16_t)0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = (uint32_t)e[2 * i] | ((uint32_t)e[2 * i + 1] << 16);
+    }
+    return out;
+}
+
+// Position of key (or query) `x` of a 16-group inside an LDS row that feeds the A operand
+// of an MFMA whose B operand comes straight from a C-layout register block: C rows
+// 8b + 4g + c (b, g in {0,1}) must sit at slot 8g + 4b + c, i.e. bits 2 and 3 swap.
+__device__ __forceinline__ int slot_of(int x) {
+    return (x & ~12) | ((x & 4) << 1) | ((x & 8) >> 1);
+}
+
+// Grid id -> logical work id such that the workgroups that land on one XCD (hardware hands
+// consecutive ids to the 8 XCDs round-robin) cover a contiguous range of logical ids and so
+// share K/V of the same (batch, head) in that XCD's L2.
+__device__ __forceinline__ int xcd_remap(int wg, int total) {
+    constexpr int kXcd = 8;
+    if (total % kXcd != 0) return wg;
+    return (wg % kXcd) * (total / kXcd) + wg / kXcd;
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+} // namespace fb

@@ -1,0 +1,49 @@
+// Host-visible kernel argument blocks and launchers (implemented in fb_fwd.hip / fb_bwd.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fb_device.h"
+
+namespace fb {
+
+struct FwdArgs {
+    Tensor q, k, v, qb, kb, o;
+    MaskDesc mask;
+    float *lse; // (B, H, Lq)
+    int B, H, Lq, Lk, d, r;
+    int causal;
+    float scale;
+    int ntiles_m; // query tiles per (batch, head)
+};
+
+struct BwdArgs {
+    Tensor q, k, v, qb, kb, o, dout;
+    Tensor dq, dk, dv, dqb, dkb;
+    MaskDesc mask;
+    const float *lse; // (B, H, Lq)
+    float *delta;     // (B, H, Lq)
+    float *dq_acc;    // (B*H, DQ_ROWS, Lq_pad) fp32: transposed partial sums of [dq | dq_bias]
+    int64_t lq_pad;   // row length of dq_acc
+    int dq_rows;      // rows of dq_acc per (batch, head)
+    int r_row0;       // first dq_bias row inside dq_acc (= d; rows [0, d) hold dq)
+    int B, H, Lq, Lk, d, r;
+    int causal;
+    float scale;
+    int ntiles_n; // key tiles per (batch, head)
+};
+
+// Each returns hipSuccess or the launch error.  `bf16` selects the element type.
+hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream);
+hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream);
+hipError_t launch_bwd_main(const BwdArgs &a, bool bf16, hipStream_t stream);
+hipError_t launch_bwd_finalize(const BwdArgs &a, bool bf16, hipStream_t stream);
+
+// Padded sizes the dispatchers use: d is covered by 16-wide contraction steps of the
+// QK^T product (NKD of them) and the rank by NKR more; both rounded up to the next
+// instantiated size (1, 2, 4, 8 steps).
+inline int steps_pow2(int n16) { return n16 <= 1 ? 1 : n16 <= 2 ? 2 : n16 <= 4 ? 4 : 8; }
+inline int nkd_of(int d) { return steps_pow2((d + 15) / 16); }
+inline int nkr_of(int r) { return r == 0 ? 0 : steps_pow2((r + 15) / 16); }
+
+} // namespace fb

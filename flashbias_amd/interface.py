@@ -1,0 +1,168 @@
+"""``flash_bias_func``: the reference's operator on MI355X.
+
+Mirrors ``FlashBiasFunc`` of the reference (flash_bias/flash_bias_triton.py:1345-1405): same
+name, same positional arguments and defaults, same return values, backed by the HIP kernels
+of ``libflashbias_hip.so`` through its C ABI.  PyTorch only provides device memory and the
+stream.  Differences from the reference, all on purpose:
+
+* gradients of factors that broadcast over batch or heads are summed over those
+  dimensions (the reference indexes the un-expanded tensors with expanded strides in its
+  backward, flash_bias_triton.py:1227-1231, :1364);
+* ``lse`` is (B, H, Lq), not rounded up to a multiple of 128 (:1145-1146);
+* ``softmax_scale`` of ``None`` or 0 gives ``1/sqrt(d)`` as in the reference (:1110).
+"""
+import math
+
+import torch
+
+from . import _lib
+
+
+def _tensor(x):
+    """(B, L, H, c) tensor -> FbTensor with (batch, head, seq) element strides."""
+    return _lib.FbTensor(x.data_ptr(), x.stride(0), x.stride(2), x.stride(1))
+
+
+def _dtype_code(dtype):
+    if dtype == torch.float16:
+        return _lib.FB_F16
+    if dtype == torch.bfloat16:
+        return _lib.FB_BF16
+    if dtype == torch.float32:
+        return _lib.FB_F32
+    raise TypeError(f"unsupported dtype {dtype}")
+
+
+def _last_dim_contiguous(x):
+    return x if x.stride(-1) == 1 else x.contiguous()
+
+
+def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
+    """Argument checks of _flash_attn_forward (flash_bias_triton.py:1100-1143) and the
+    parameter block shared by forward and backward.  Returns (params, keepalive)."""
+    batch, seqlen_q, nheads, d = q.shape
+    _, seqlen_k, _, _ = k.shape
+    assert k.shape == (batch, seqlen_k, nheads, d)
+    assert v.shape == (batch, seqlen_k, nheads, d)
+    assert d <= 128, "FlashBias only supports head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda
+    p = _lib.new_params()
+    p.dtype = _dtype_code(q.dtype)
+    p.B, p.H, p.Lq, p.Lk, p.d = batch, nheads, seqlen_q, seqlen_k, d
+    p.causal = int(bool(causal))
+    p.scale = softmax_scale or 1.0 / math.sqrt(d)
+    p.q, p.k, p.v = _tensor(q), _tensor(k), _tensor(v)
+    keep = []
+    if q_bias is not None:
+        assert k_bias is not None and q_bias.dtype == k_bias.dtype == q.dtype
+        assert q_bias.is_cuda and k_bias.is_cuda
+        rank = q_bias.shape[-1]
+        assert k_bias.shape[-1] == rank
+        # stride-0 broadcast over batch / heads (:1135-1136)
+        qbe = q_bias.expand(batch, seqlen_q, nheads, rank)
+        kbe = k_bias.expand(batch, seqlen_k, nheads, rank)
+        p.r = rank
+        p.q_bias, p.k_bias = _tensor(qbe), _tensor(kbe)
+        keep += [qbe, kbe]
+    if mask is not None:
+        assert mask.dtype in (q.dtype, torch.float)
+        assert mask.is_cuda
+        assert mask.dim() == 4
+        if mask.stride(-1) != 1:
+            mask = mask.contiguous()
+        if mask.shape[2:] == (1, seqlen_k):
+            p.mask_type = _lib.FB_MASK_VECTOR
+        elif mask.shape[2:] == (seqlen_q, seqlen_k):
+            p.mask_type = _lib.FB_MASK_MATRIX
+        else:
+            raise RuntimeError("Last 2 dimensions of mask must be (1, seqlen_k) or (seqlen_q, seqlen_k)")
+        me = mask.expand(batch, nheads, seqlen_q, seqlen_k)
+        p.mask = _lib.FbTensor(me.data_ptr(), me.stride(0), me.stride(1), me.stride(2))
+        p.mask_dtype = _dtype_code(mask.dtype)
+        keep.append(me)
+    return p, keep
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
+    lib = _lib.load()
+    p, keep = _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+    o = torch.empty_like(q)
+    lse = torch.empty((p.B, p.H, p.Lq), device=q.device, dtype=torch.float32)
+    p.o, p.lse = _tensor(o), lse.data_ptr()
+    with torch.cuda.device(q.device):
+        _lib.check_status(lib.fb_fwd(p, _stream()))
+    del keep
+    return o, lse, p.scale
+
+
+def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale):
+    lib = _lib.load()
+    do = _last_dim_contiguous(do)
+    p, keep = _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    p.o, p.lse, p.dout = _tensor(o), lse.data_ptr(), _tensor(do)
+    p.dq, p.dk, p.dv = _tensor(dq), _tensor(dk), _tensor(dv)
+    dqb_full = dkb_full = None
+    if q_bias is not None:
+        dqb_full = torch.empty((p.B, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
+        dkb_full = torch.empty((p.B, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
+        p.dq_bias, p.dk_bias = _tensor(dqb_full), _tensor(dkb_full)
+    delta = torch.empty_like(lse)
+    nbytes = lib.fb_bwd_workspace_bytes(p)
+    workspace = torch.empty(nbytes // 4, device=q.device, dtype=torch.float32)
+    p.delta, p.workspace, p.workspace_bytes = delta.data_ptr(), workspace.data_ptr(), nbytes
+    with torch.cuda.device(q.device):
+        _lib.check_status(lib.fb_bwd(p, _stream()))
+    del keep
+    dq_bias = dk_bias = None
+    if q_bias is not None:
+        dq_bias = _reduce_like(dqb_full, q_bias)
+        dk_bias = _reduce_like(dkb_full, k_bias)
+    return dq, dk, dv, dq_bias, dk_bias
+
+
+def _reduce_like(full, ref):
+    """Sum a full (B, L, H, r) gradient over the dims in which ``ref`` was broadcast."""
+    dims = [i for i in (0, 2) if ref.shape[i] == 1 and full.shape[i] != 1]
+    if dims:
+        full = full.sum(dim=dims, keepdim=True, dtype=torch.float32).to(ref.dtype)
+    return full
+
+
+class FlashBiasFunc(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, q_bias=None, k_bias=None, mask=None, causal=False, softmax_scale=None):
+        """
+        q: (batch_size, seqlen_q, nheads, headdim)
+        k, v: (batch_size, seqlen_k, nheads, headdim)
+        q_bias: (batch_size | 1, seqlen_q, nheads | 1, rankdim)
+        k_bias: (batch_size | 1, seqlen_k, nheads | 1, rankdim)
+        mask: optional additive mask broadcastable to (batch, nheads, seqlen_q, seqlen_k) whose
+            last two dims are (1, seqlen_k) or (seqlen_q, seqlen_k); receives no gradient
+        softmax_scale: multiplies q k^T only; defaults to 1 / sqrt(headdim)
+        """
+        if q_bias is not None:
+            q, k, v, q_bias, k_bias = [_last_dim_contiguous(x) for x in (q, k, v, q_bias, k_bias)]
+        else:
+            q, k, v = [_last_dim_contiguous(x) for x in (q, k, v)]
+        o, lse, ctx.softmax_scale = _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+        ctx.save_for_backward(q, k, v, o, q_bias, k_bias, lse, mask)
+        ctx.causal = causal
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, q_bias, k_bias, lse, mask = ctx.saved_tensors
+        assert not ctx.needs_input_grad[5], "FlashBias does not support mask gradient yet"
+        dq, dk, dv, dq_bias, dk_bias = _flash_bias_backward(
+            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale)
+        return dq, dk, dv, dq_bias, dk_bias, None, None, None
+
+
+flash_bias_func = FlashBiasFunc.apply

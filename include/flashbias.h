@@ -1,0 +1,123 @@
+/*
+ * flashbias.h -- C ABI of the MI355X (gfx950) FlashBias attention library.
+ *
+ * The library is the device side of the reference's operator
+ *     flash_bias_func(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+ * (flash_bias/flash_bias_triton.py:1345-1405).  Each entry point below names the reference
+ * function it replaces.  Conventions shared by all of them:
+ *
+ *   - Nothing here allocates or frees device memory: every buffer, including scratch
+ *     (lse, delta, the backward workspace), is owned by the caller, as in the reference where
+ *     torch allocates o/lse/tmp/delta/dq_accum (flash_bias_triton.py:1145-1148, :1212-1219).
+ *   - Launches are asynchronous on the given hipStream_t (passed as void*); no global
+ *     mutable state, no autotuning side effects.
+ *   - Return value: FB_OK (0) or a negative fb_status; fb_last_error() gives the text of the
+ *     last failure on the calling thread.  No C++ exception crosses the boundary.
+ *   - Tensors use the reference layout (batch, seq, heads, channels) with the channel
+ *     dimension contiguous; batch / head / seq are addressed through element strides, the
+ *     way the Triton launchers pass them (flash_bias_triton.py:1163-1177).
+ */
+#ifndef FLASHBIAS_H
+#define FLASHBIAS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FB_VERSION 1
+#define FB_MAX_HEADDIM 128 /* flash_bias_triton.py:1106 */
+#define FB_MAX_RANK 128
+
+typedef enum fb_status {
+    FB_OK = 0,
+    FB_ERR_NULL = -1,       /* required pointer missing */
+    FB_ERR_SHAPE = -2,      /* non-positive size, d > 128, r > 128 */
+    FB_ERR_DTYPE = -3,      /* only fp16 / bf16 inputs (flash_bias_triton.py:1108) */
+    FB_ERR_STRIDE = -4,     /* stride would alias gradient rows / negative stride */
+    FB_ERR_MASK = -5,       /* bad mask type / dtype */
+    FB_ERR_WORKSPACE = -6,  /* workspace missing or too small */
+    FB_ERR_ABI = -7,        /* fb_params.size does not match this library */
+    FB_ERR_LAUNCH = -8,     /* HIP reported a launch error */
+    FB_ERR_SCALE = -9       /* softmax scale not finite / not positive */
+} fb_status;
+
+typedef enum fb_dtype { FB_F16 = 0, FB_BF16 = 1, FB_F32 = 2 /* mask only */ } fb_dtype;
+
+/* flash_bias_triton.py:1112-1123 */
+typedef enum fb_mask_type { FB_MASK_NONE = 0, FB_MASK_VECTOR = 1, FB_MASK_MATRIX = 2 } fb_mask_type;
+
+/* A (batch, seq, heads, channels) tensor with contiguous channels.  Strides are in elements.
+ * For the mask, which is (batch, heads, Lq|1, Lk), stride_s is the stride of the query row
+ * (0 for the vector type) and stride_b / stride_h may be 0 (broadcast). */
+typedef struct fb_tensor {
+    void *ptr;
+    int64_t stride_b, stride_h, stride_s;
+} fb_tensor;
+
+typedef struct fb_params {
+    uint32_t size; /* sizeof(fb_params) as seen by the caller */
+    int32_t dtype; /* fb_dtype of q, k, v, factors, o and all gradients */
+    int32_t B, H, Lq, Lk;
+    int32_t d;     /* head dim, 1..128 */
+    int32_t r;     /* bias rank, 0 = no factors (plain attention, flash_bias_triton.py:1359) */
+    int32_t causal;     /* top-left aligned: key j visible from query i iff j <= i (:262) */
+    int32_t mask_type;  /* fb_mask_type */
+    int32_t mask_dtype; /* dtype or FB_F32 (:1115) */
+    float scale;        /* softmax scale, applied to q k^T only, never to the bias (:248) */
+
+    fb_tensor q, k, v;        /* in */
+    fb_tensor q_bias, k_bias; /* in; stride_b / stride_h = 0 broadcasts (:1135-1136) */
+    fb_tensor mask;           /* in, additive, no gradient (:1371) */
+    fb_tensor o;              /* fwd: out; bwd: in */
+    float *lse;               /* (B, H, Lq) fp32, natural log; fwd: out; bwd: in (:323) */
+
+    fb_tensor dout;             /* bwd in: upstream gradient of o */
+    fb_tensor dq, dk, dv;       /* bwd out */
+    fb_tensor dq_bias, dk_bias; /* bwd out, full (B, L, H, r) shape: the caller reduces over
+                                   broadcast dims */
+    float *delta;               /* (B, H, Lq) fp32 scratch, written by the backward */
+    void *workspace;            /* fb_bwd_workspace_bytes() of device memory */
+    uint64_t workspace_bytes;
+} fb_params;
+
+/* Library / ABI version. */
+int fb_version(void);
+
+/* Text of the last error on this thread ("" if none). */
+const char *fb_last_error(void);
+
+/* Argument checks of _flash_attn_forward / _flash_attn_backward
+ * (flash_bias_triton.py:1102-1129, :1201-1225) without touching the GPU.
+ * pass: 0 = forward, 1 = backward. */
+int fb_check(const fb_params *p, int pass);
+
+/* Replaces _flash_attn_forward + _fwd_kernel (flash_bias_triton.py:1100-1194, :62-355):
+ * o = softmax(scale q k^T + q_bias k_bias^T + mask) v and lse. */
+int fb_fwd(const fb_params *p, void *stream);
+
+/* Bytes of device scratch the backward needs for these sizes (the reference's dq_accum /
+ * dq_bias_accum, flash_bias_triton.py:1212-1219). */
+uint64_t fb_bwd_workspace_bytes(const fb_params *p);
+
+/* Replaces _flash_attn_backward (flash_bias_triton.py:1197-1342): runs the three phases
+ * below in order on the stream. */
+int fb_bwd(const fb_params *p, void *stream);
+
+/* The phases of fb_bwd, exported so that a harness can time them separately.
+ *   fb_bwd_preprocess: delta = rowsum(o * dout) and zero the workspace
+ *                      (_bwd_preprocess_do_o_dot, :358-400; init_to_zero, :872-879)
+ *   fb_bwd_main:       recompute P from lse; dk, dv, dk_bias; dq / dq_bias partial sums
+ *                      into the workspace (_bwd_kernel, :882-1097; :450-869)
+ *   fb_bwd_finalize:   workspace -> dq (times scale) and dq_bias in the input dtype
+ *                      (dq.copy_(dq_accum), :1340-1342) */
+int fb_bwd_preprocess(const fb_params *p, void *stream);
+int fb_bwd_main(const fb_params *p, void *stream);
+int fb_bwd_finalize(const fb_params *p, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHBIAS_H */
