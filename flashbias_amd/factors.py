@@ -1,0 +1,73 @@
+"""Builders of the low-rank bias factors that feed ``flash_bias_func``.
+
+Three ways to obtain ``q_bias`` / ``k_bias`` with ``q_bias @ k_bias^T == bias``:
+exact closed forms (ALiBi, squared spatial distance), and a truncated SVD of a learned bias
+table (Swin-V2 relative position bias).  All factors come back in the operator's layout
+(B | 1, L, H | 1, r).
+"""
+import math
+
+import torch
+
+
+def alibi_slopes(nheads):
+    """Per-head slope m_h = 2^(-8 (h+1) / H) (1_Language_Model/attention_with_alibi_bias.py:8-15)."""
+    h = torch.arange(1, nheads + 1, dtype=torch.float64)
+    return torch.pow(2.0, -8.0 * h / nheads).float()
+
+
+def alibi_factors(seqlen_q, seqlen_k, nheads, dtype=torch.float32, device=None):
+    """Exact rank-2 factors of the ALiBi bias  -m_h (i - j):
+    q_bias[i] = [-m_h i, 1],  k_bias[j] = [1, m_h j].
+    (The demo module of the reference, attention_with_alibi_bias.py:49-52, uses the opposite
+    sign; this is the standard ALiBi penalty.)  Computed in fp32, cast once."""
+    m = alibi_slopes(nheads).to(device)
+    i = torch.arange(seqlen_q, dtype=torch.float32, device=device)
+    j = torch.arange(seqlen_k, dtype=torch.float32, device=device)
+    q_bias = torch.stack([-(i[:, None] * m[None, :]), torch.ones(seqlen_q, nheads, device=device)], dim=-1)
+    k_bias = torch.stack([torch.ones(seqlen_k, nheads, device=device), j[:, None] * m[None, :]], dim=-1)
+    return q_bias[None].to(dtype), k_bias[None].to(dtype)
+
+
+def distance_factors(x_q, x_k, alpha, dtype=torch.float32):
+    """Exact rank-(D+2) factors of  -alpha |x_i - x_j|^2  for points x (B, N, D):
+    q_bias = [-alpha |x_i|^2, -alpha, 2 alpha x_i],  k_bias = [1, |x_j|^2, x_j]
+    (the spatial-distance decomposition of the paper, pic/exact_decompose_pde.png).
+    Shapes (B, N, 1, D + 2): shared by all heads."""
+    nq = (x_q * x_q).sum(-1, keepdim=True)
+    nk = (x_k * x_k).sum(-1, keepdim=True)
+    q_bias = torch.cat([-alpha * nq, torch.full_like(nq, -alpha), 2.0 * alpha * x_q], dim=-1)
+    k_bias = torch.cat([torch.ones_like(nk), nk, x_k], dim=-1)
+    return q_bias[:, :, None, :].to(dtype), k_bias[:, :, None, :].to(dtype)
+
+
+def svd_factors(bias, rank, dtype=torch.float32):
+    """Best rank-``rank`` factors (Eckart-Young) of a per-head bias table (H, Lq, Lk).
+    Returns q_bias (1, Lq, H, rank), k_bias (1, Lk, H, rank) and the relative Frobenius error
+    of the reconstruction, ``|bias - q_bias k_bias^T|_F / |bias|_F``, per head."""
+    u, s, vh = torch.linalg.svd(bias.double(), full_matrices=False)
+    root = s[:, :rank].sqrt()
+    q_bias = u[:, :, :rank] * root[:, None, :]
+    k_bias = vh[:, :rank, :].transpose(1, 2) * root[:, None, :]
+    tail = (s[:, rank:] ** 2).sum(-1).sqrt()
+    rel = tail / (s ** 2).sum(-1).sqrt()
+    return (q_bias.permute(1, 0, 2)[None].to(dtype).contiguous(),
+            k_bias.permute(1, 0, 2)[None].to(dtype).contiguous(), rel.float())
+
+
+def swin_v2_bias_table(window, nheads, seed=0, hidden=512):
+    """A Swin-V2 style continuous relative position bias (H, N, N) for a ``window`` x ``window``
+    token grid with a randomly initialised 2 -> hidden -> H ReLU MLP on log-spaced relative
+    coordinates, squashed to (0, 16) (2_Vision_Transformer/swin_transformer_v2.py:98-131)."""
+    g = torch.Generator().manual_seed(seed)
+    w1 = (torch.rand(hidden, 2, generator=g) * 2 - 1) / math.sqrt(2.0)
+    b1 = (torch.rand(hidden, generator=g) * 2 - 1) / math.sqrt(2.0)
+    w2 = (torch.rand(nheads, hidden, generator=g) * 2 - 1) / math.sqrt(hidden)
+    rel = torch.arange(-(window - 1), window, dtype=torch.float32) / max(window - 1, 1) * 8.0
+    rel = torch.sign(rel) * torch.log2(rel.abs() + 1.0) / math.log2(8.0)
+    table = torch.stack(torch.meshgrid(rel, rel, indexing="ij"), dim=-1)  # (2W-1, 2W-1, 2)
+    table = torch.relu(table @ w1.t() + b1) @ w2.t()  # (2W-1, 2W-1, H)
+    pos = torch.stack(torch.meshgrid(torch.arange(window), torch.arange(window), indexing="ij")).flatten(1)
+    diff = pos[:, :, None] - pos[:, None, :] + (window - 1)  # (2, N, N), each in [0, 2W-2]
+    bias = table[diff[0], diff[1]]  # (N, N, H)
+    return 16.0 * torch.sigmoid(bias.permute(2, 0, 1)).contiguous()

@@ -143,3 +143,45 @@ def flashbias_concat_sdpa(q, k, v, q_bias, k_bias, softmax_scale, causal=False):
     out = torch.nn.functional.scaled_dot_product_attention(
         qc, kc, v.transpose(1, 2), attn_mask=None, dropout_p=0.0, is_causal=causal, scale=1.0)
     return out.transpose(1, 2)
+
+
+def flashbias_backward_stored(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, o, lse, do,
+                              round_dtype=None, dtype=torch.float32):
+    """Backward from the *stored* forward results, the contract of the reference's
+    ``_flash_attn_backward(do, q, k, v, o, ..., lse, ...)`` (flash_bias_triton.py:1197):
+
+        delta = rowsum(o * do)                     (:398, o as stored in the input dtype)
+        P     = exp(S - lse)                       (:670)
+        dV    = round(P)^T dO                      (:696-697)
+        dP    = dO V^T                             (:705)
+        dS    = round(P * (dP - delta))            (:714)
+        dK = scale dS^T Q, dK_b = dS^T Q_b         (:717-719)
+        dQ = scale dS K,   dQ_b = dS K_b           (:728-732)
+
+    ``round_dtype`` (fp16 / bf16) applies the two roundings the reference applies before its
+    matmuls; ``None`` keeps everything in ``dtype`` and then this equals autograd through the
+    eager path when (o, lse) are the eager ones.  Factor gradients are reduced over broadcast
+    dims.  Returns (dq, dk, dv, dq_bias, dk_bias)."""
+    scale = softmax_scale or default_scale(q.shape[-1])
+    batch, _, nheads, _ = q.shape
+    rnd = (lambda t: t.to(round_dtype).to(dtype)) if round_dtype is not None else (lambda t: t)
+    qh, kh, vh, doh, oh = (t.to(dtype).permute(0, 2, 1, 3) for t in (q, k, v, do, o))
+    bias = _dense_bias(q.to(dtype), None if q_bias is None else q_bias.to(dtype),
+                       None if k_bias is None else k_bias.to(dtype), mask)
+    s = logits(q.to(dtype), k.to(dtype), scale, bias, causal).permute(0, 2, 1, 3)
+    p = torch.exp(s - lse.to(dtype)[..., None])
+    delta = (oh * doh).sum(-1, keepdim=True)
+    dv = rnd(p).transpose(-1, -2) @ doh
+    ds = rnd(p * (doh @ vh.transpose(-1, -2) - delta))
+    dq = scale * (ds @ kh)
+    dk = scale * (ds.transpose(-1, -2) @ qh)
+    out = [t.permute(0, 2, 1, 3) for t in (dq, dk, dv)]
+    if q_bias is None:
+        return tuple(out) + (None, None)
+    qbh = q_bias.to(dtype).expand(batch, -1, nheads, -1).permute(0, 2, 1, 3)
+    kbh = k_bias.to(dtype).expand(batch, -1, nheads, -1).permute(0, 2, 1, 3)
+    for g, ref in ((ds @ kbh, q_bias), (ds.transpose(-1, -2) @ qbh, k_bias)):
+        g = g.permute(0, 2, 1, 3)
+        dims = [i for i in (0, 2) if ref.shape[i] == 1 and g.shape[i] != 1]
+        out.append(g.sum(dim=dims, keepdim=True) if dims else g)
+    return tuple(out)

@@ -1,0 +1,137 @@
+"""CPU-only checks of the C ABI: the in-tree library loads, exports every symbol that
+include/flashbias.h declares, and rejects bad arguments with the documented status codes
+before anything touches a GPU."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from flashbias_amd import _lib, flash_bias_func
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "flashbias.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(fb_[a-z_]+)\s*\(", text))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert declared == set(_lib.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.fb_version() == 1
+
+
+def _good(pass_=0):
+    p = _lib.new_params()
+    p.dtype = _lib.FB_BF16
+    p.B, p.H, p.Lq, p.Lk, p.d, p.r = 2, 4, 128, 128, 32, 8
+    p.scale = 0.25
+    fake = 0x10000  # never dereferenced: fb_check does not touch the GPU
+    t = lambda c: _lib.FbTensor(fake, 128 * 4 * c, c, 4 * c)
+    p.q, p.k, p.v, p.o = t(32), t(32), t(32), t(32)
+    p.q_bias, p.k_bias = t(8), t(8)
+    p.lse = fake
+    if pass_ == 1:
+        p.dout, p.dq, p.dk, p.dv = t(32), t(32), t(32), t(32)
+        p.dq_bias, p.dk_bias = t(8), t(8)
+        p.delta = fake
+        p.workspace = fake
+        p.workspace_bytes = _lib.load().fb_bwd_workspace_bytes(p)
+    return p
+
+
+def test_check_accepts_good_params():
+    lib = _lib.load()
+    assert lib.fb_check(_good(0), 0) == 0
+    assert lib.fb_check(_good(1), 1) == 0
+    assert lib.fb_last_error() == b""
+
+
+def test_workspace_size_formula():
+    p = _good(1)
+    # (B*H) * (d + r) rows of round_up(Lq, 32) fp32 partial sums
+    assert _lib.load().fb_bwd_workspace_bytes(p) == 2 * 4 * (32 + 8) * 128 * 4
+    p.Lq = 100
+    assert _lib.load().fb_bwd_workspace_bytes(p) == 2 * 4 * (32 + 8) * 128 * 4
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda p: setattr(p, "size", 8), -7),
+    (lambda p: setattr(p, "dtype", 2), -3),
+    (lambda p: setattr(p, "d", 129), -2),
+    (lambda p: setattr(p, "d", 0), -2),
+    (lambda p: setattr(p, "r", 129), -2),
+    (lambda p: setattr(p, "Lk", 0), -2),
+    (lambda p: setattr(p, "scale", 0.0), -9),
+    (lambda p: setattr(p, "scale", float("nan")), -9),
+    (lambda p: setattr(p.q, "ptr", None), -1),
+    (lambda p: setattr(p.k_bias, "ptr", None), -1),
+    (lambda p: setattr(p, "lse", None), -1),
+    (lambda p: setattr(p.v, "stride_s", -32), -4),
+    (lambda p: setattr(p.o, "stride_b", 0), -4),
+    (lambda p: setattr(p.o, "stride_s", 16), -4),
+    (lambda p: setattr(p, "mask_type", 3), -5),
+    (lambda p: (setattr(p, "mask_type", 1), setattr(p, "mask_dtype", 0), setattr(p.mask, "ptr", 0x10000)), -5),
+    (lambda p: (setattr(p, "mask_type", 2), setattr(p, "mask_dtype", 2)), -1),
+])
+def test_check_rejects_forward(mutate, code):
+    p = _good(0)
+    mutate(p)
+    lib = _lib.load()
+    assert lib.fb_check(p, 0) == code
+    assert lib.fb_last_error() != b""
+    assert lib.fb_fwd(p, None) == code  # rejected before any launch
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda p: setattr(p.dout, "ptr", None), -1),
+    (lambda p: setattr(p.dq_bias, "ptr", None), -1),
+    (lambda p: setattr(p, "delta", None), -1),
+    (lambda p: setattr(p.dk, "stride_h", 0), -4),
+    (lambda p: setattr(p.dk_bias, "stride_b", 0), -4),
+    (lambda p: setattr(p, "workspace", None), -6),
+    (lambda p: setattr(p, "workspace_bytes", 16), -6),
+    (lambda p: setattr(p, "workspace", 0x10004), -6),
+])
+def test_check_rejects_backward(mutate, code):
+    p = _good(1)
+    mutate(p)
+    lib = _lib.load()
+    assert lib.fb_check(p, 1) == code
+    for fn in (lib.fb_bwd, lib.fb_bwd_preprocess, lib.fb_bwd_main, lib.fb_bwd_finalize):
+        assert fn(p, None) == code
+
+
+def test_null_params():
+    lib = _lib.load()
+    assert lib.fb_check(None, 0) == -1
+    assert lib.fb_bwd_workspace_bytes(None) == 0
+
+
+def test_params_struct_matches_header_size():
+    # a wrong field order or type would change the size the library checks against
+    p = _lib.new_params()
+    assert p.size == ctypes.sizeof(_lib.FbParams)
+    p.B = p.H = p.Lq = p.Lk = p.d = 1
+    p.scale = 1.0
+    assert _lib.load().fb_check(p, 0) == -1  # got past the ABI check, stopped at "q: null"
+    assert b"q:" in _lib.load().fb_last_error()
+
+
+def test_operator_rejects_cpu_and_fp32_inputs():
+    """No CPU or fallback path: the host wrapper asserts like the reference's launcher
+    (flash_bias/flash_bias_triton.py:1107-1109)."""
+    q = torch.randn(1, 8, 1, 16, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError):
+        flash_bias_func(q, q, q)
+    with pytest.raises(AssertionError):
+        flash_bias_func(q.float(), q.float(), q.float())
+    with pytest.raises(AssertionError):
+        flash_bias_func(q, q[:, :4], q)

@@ -1,0 +1,316 @@
+"""GPU parity tests: the HIP path, called through the C ABI by ``flash_bias_func``, against
+the CPU oracle on the same seeded, dtype-rounded inputs.
+
+Tolerances (the gate of the headline metric): max-abs error of o <= 1e-2 (fp16) / 2e-2 (bf16);
+for each of dq, dk, dv, dq_bias, dk_bias: max|err| / max|ref| <= 5e-2; causal structure exact.
+"""
+import math
+
+import pytest
+import torch
+
+from _util import GRAD_TOL, O_TOL, errors, make_inputs, oracle, run_gpu
+from flashbias_amd import flash_bias_func, workloads
+
+pytestmark = pytest.mark.gpu
+NAMES = ("o", "dq", "dk", "dv", "dq_bias", "dk_bias")
+
+
+def _gate(got, ref, dtype, skip=()):
+    refs = [ref[0]] + list(ref[2:])
+    for name, g, w in zip(NAMES, got, refs):
+        if w is None:
+            assert g is None
+            continue
+        assert g.shape == w.shape, name
+        assert torch.isfinite(g).all(), name
+        err, rel = errors(g, w)
+        if name == "o":
+            assert err <= O_TOL[dtype], (name, err)
+        elif w.abs().max() == 0:  # e.g. a single visible key: dS is identically zero
+            assert err <= 1e-5, (name, err)
+        elif name not in skip:
+            assert rel <= GRAD_TOL, (name, err, rel)
+
+
+def _case(gpu_device, B, Lq, Lk, H, d, r, dtype, causal, mask=None, scale=None, seed=1, **bc):
+    q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, dtype, seed=seed, **bc)
+    ref = oracle(q, k, v, qb, kb, mask, causal, scale, do)
+    got = run_gpu(flash_bias_func, q, k, v, qb, kb, mask, causal, scale, do, gpu_device)
+    _gate(got, ref, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_benchmark_shape_family(gpu_device, dtype, causal):
+    """B2 H4 d32 r8 of flash_bias/config.py:12 at L=1024 (also the reference's own
+    correctness shape family, flash_bias/benchmark.py:31)."""
+    _case(gpu_device, 2, 1024, 1024, 4, 32, 8, dtype, causal)
+
+
+def test_reference_correctness_script_shape(gpu_device):
+    """flash_bias/benchmark.py:27-47,65: B1 L1024 H2 d32 r8 fp16, factors ~ N(0,1) (not scaled),
+    upstream gradient of loss = -o.sum()."""
+    g = torch.Generator().manual_seed(0)
+    q, k, v = [torch.randn(1, 1024, 2, 32, generator=g).half() for _ in range(3)]
+    qb, kb = [torch.randn(1, 1024, 2, 8, generator=g).half() for _ in range(2)]
+    do = -torch.ones(1, 1024, 2, 32).half()
+    ref = oracle(q, k, v, qb, kb, None, False, 1 / math.sqrt(32), do)
+    got = run_gpu(flash_bias_func, q, k, v, qb, kb, None, False, 1 / math.sqrt(32), do, gpu_device)
+    _gate(got, ref, torch.float16)
+
+
+@pytest.mark.parametrize("d", [16, 32, 40, 64, 128])
+@pytest.mark.parametrize("causal", [False, True])
+def test_head_dims(gpu_device, d, causal):
+    _case(gpu_device, 1, 200, 200, 2, d, 8, torch.bfloat16, causal)
+
+
+@pytest.mark.parametrize("r", [0, 2, 5, 8, 16, 32, 96])
+def test_ranks(gpu_device, r):
+    _case(gpu_device, 1, 160, 224, 2, 32, r, torch.bfloat16, False)
+
+
+@pytest.mark.parametrize("Lq,Lk", [(1, 1), (1, 257), (75, 117), (117, 75), (129, 64), (64, 129), (255, 255)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_ragged_lengths(gpu_device, Lq, Lk, causal):
+    _case(gpu_device, 2, Lq, Lk, 3, 40, 5, torch.float16, causal)
+
+
+def test_odd_head_dim_and_unaligned_rank(gpu_device):
+    """d and r that are not multiples of 8: rows are not 16-byte aligned, the element-wise
+    load path is used."""
+    _case(gpu_device, 2, 90, 70, 2, 20, 3, torch.bfloat16, True)
+    _case(gpu_device, 1, 130, 130, 3, 100, 7, torch.float16, False)
+
+
+@pytest.mark.parametrize("bq,bk", [((True, False), (True, False)), ((True, True), (False, True)),
+                                   ((False, True), (True, True))])
+def test_broadcast_factors(gpu_device, bq, bk):
+    """Factors shared over batch and/or heads (stride 0); their gradients are summed over the
+    shared dims, which is what autograd through the eager path gives."""
+    _case(gpu_device, 3, 100, 140, 4, 32, 16, torch.bfloat16, False, bq=bq, bk=bk)
+
+
+@pytest.mark.parametrize("kind", ["vector", "matrix", "matrix_bcast", "vector_f32"])
+@pytest.mark.parametrize("causal", [False, True])
+def test_additive_mask(gpu_device, kind, causal):
+    B, Lq, Lk, H = 2, 96, 150, 3
+    g = torch.Generator().manual_seed(5)
+    if kind == "vector":
+        mask = torch.randn(B, 1, 1, Lk, generator=g).bfloat16()
+    elif kind == "vector_f32":
+        mask = torch.randn(B, H, 1, Lk, generator=g)
+    elif kind == "matrix":
+        mask = torch.randn(B, H, Lq, Lk, generator=g).bfloat16()
+    else:  # the Swin shifted-window form: 0 / -100 per (window, 1, N, N)
+        mask = (torch.rand(B, 1, Lq, Lk, generator=g) < 0.3).float() * -100.0
+    _case(gpu_device, B, Lq, Lk, H, 32, 8, torch.bfloat16, causal, mask=mask)
+
+
+def test_noncontiguous_inputs_and_scale(gpu_device):
+    """q, k, v as strided views of a packed qkv projection, as the application modules create
+    them; non-default softmax scale."""
+    B, L, H, d, r = 2, 130, 4, 32, 8
+    g = torch.Generator().manual_seed(9)
+    qkv = torch.randn(B, L, 3, H, d, generator=g).bfloat16()
+    q, k, v = qkv[:, :, 0], qkv[:, :, 1], qkv[:, :, 2]
+    qb = (torch.randn(B, H, L, r, generator=g) / math.sqrt(r)).bfloat16().permute(0, 2, 1, 3)
+    kb = (torch.randn(B, H, L, r, generator=g) / math.sqrt(r)).bfloat16().permute(0, 2, 1, 3)
+    do = torch.randn(B, L, H, d, generator=g).bfloat16()
+    ref = oracle(q, k, v, qb, kb, None, False, 0.3, do)
+    dev = gpu_device
+    qkv_d = qkv.to(dev).requires_grad_(True)
+    qb_d = qb.to(dev).requires_grad_(True)  # keeps the permuted strides
+    kb_d = kb.to(dev).requires_grad_(True)
+    assert qb_d.stride(-1) == 1 and not qb_d.is_contiguous()
+    o = flash_bias_func(qkv_d[:, :, 0], qkv_d[:, :, 1], qkv_d[:, :, 2], qb_d, kb_d, None, False, 0.3)
+    gqkv, gqb, gkb = torch.autograd.grad(o, [qkv_d, qb_d, kb_d], do.to(dev))
+    got = [o.detach().float().cpu(), gqkv[:, :, 0].float().cpu(), gqkv[:, :, 1].float().cpu(),
+           gqkv[:, :, 2].float().cpu(), gqb.float().cpu(), gkb.float().cpu()]
+    _gate(got, ref, torch.bfloat16)
+
+
+def test_lse_and_default_scale(gpu_device):
+    from flashbias_amd.interface import _flash_bias_forward
+    q, k, v, qb, kb, do = make_inputs(2, 300, 260, 2, 64, 8, torch.bfloat16, seed=3)
+    ref = oracle(q, k, v, qb, kb, None, True, None, do)
+    dev = gpu_device
+    o, lse, scale = _flash_bias_forward(q.to(dev), k.to(dev), v.to(dev), qb.to(dev), kb.to(dev), None, True, None)
+    assert scale == pytest.approx(1 / 8)
+    assert lse.shape == (2, 2, 300) and lse.dtype == torch.float32
+    assert (lse.cpu() - ref[1]).abs().max() < 2e-3
+    o0, _, scale0 = _flash_bias_forward(q.to(dev), k.to(dev), v.to(dev), qb.to(dev), kb.to(dev), None, True, 0)
+    assert scale0 == scale and torch.equal(o0, o)  # 0 falls back to the default like `or` does
+
+
+def test_causal_structure_is_exact(gpu_device):
+    """o[:, 0] == v[:, 0] bit for bit, and changing k / v / k_bias at keys j > i leaves o[i]
+    bit-identical (top-left aligned causal mask, flash_bias_triton.py:262)."""
+    dev = gpu_device
+    q, k, v, qb, kb, _ = [t.to(dev) if t is not None else None
+                          for t in make_inputs(2, 333, 333, 3, 32, 8, torch.bfloat16, seed=4)]
+    o = flash_bias_func(q, k, v, qb, kb, None, True, None)
+    assert torch.equal(o[:, 0], v[:, 0])
+    for cut in (1, 64, 65, 200, 332):
+        k2, v2, kb2 = k.clone(), v.clone(), kb.clone()
+        k2[:, cut:] += 3
+        v2[:, cut:] -= 5
+        kb2[:, cut:] *= -2
+        o2 = flash_bias_func(q, k2, v2, qb, kb2, None, True, None)
+        assert torch.equal(o[:, :cut], o2[:, :cut]), cut
+        assert not torch.equal(o[:, cut:], o2[:, cut:]), cut
+
+
+def test_backward_reproducibility(gpu_device):
+    """dk, dv, dk_bias are accumulated in registers in a fixed order: bit-identical from run to
+    run.  dq / dq_bias go through fp32 atomics: equal up to summation order."""
+    dev = gpu_device
+    ins = [t.to(dev).requires_grad_(True) for t in make_inputs(2, 700, 700, 4, 32, 8, torch.bfloat16, seed=6)[:5]]
+    do = torch.randn(2, 700, 4, 32, device=dev, dtype=torch.bfloat16)
+    runs = []
+    for _ in range(3):
+        o = flash_bias_func(*ins, None, True, None)
+        runs.append(torch.autograd.grad(o, ins, do))
+    for other in runs[1:]:
+        for idx in (1, 2, 4):
+            assert torch.equal(runs[0][idx], other[idx])
+        for idx in (0, 3):
+            assert (runs[0][idx].float() - other[idx].float()).abs().max() <= 2e-2 * runs[0][idx].float().abs().max()
+
+
+# ------------------------------------------------------------------ named workloads (reduced)
+def _run_workload(gpu_device, w, dtype, skip=()):
+    ref = oracle(w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], None, w["causal"], w["softmax_scale"], w["do"])
+    got = run_gpu(flash_bias_func, w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], None, w["causal"],
+                  w["softmax_scale"], w["do"], gpu_device)
+    _gate(got, ref, dtype, skip)
+    return got, ref
+
+
+def _factor_grad_noise_gate(w, got, ref, dtype):
+    """Gate for dq_bias / dk_bias when the factors are large functions of position (ALiBi:
+    |k_bias| ~ m j reaches ~900).  Any flash backward that keeps o, P and dS in a 16-bit type
+    -- the reference rounds them at flash_bias_triton.py:346, :696, :714 -- amplifies that
+    rounding by |factor|: through dS directly, and through delta = rowsum(o * dO) (:398),
+    whose error e_i enters as -P_ij e_i.  Two correct implementations of the same scheme then
+    differ by a good fraction of the gradient itself.  The gate is six standard deviations of
+    that noise (each rounding uniform within +-u|x|, u = half an ulp) on top of the usual
+    5e-2 of max|ref|."""
+    from oracle import eager
+    u = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    q, k, v, do = (w[n].float() for n in ("q", "k", "v", "do"))
+    B, _, H, _ = q.shape
+    qb = w["q_bias"].float().expand(B, -1, H, -1).permute(0, 2, 1, 3)
+    kb = w["k_bias"].float().expand(B, -1, H, -1).permute(0, 2, 1, 3)
+    bias = qb @ kb.transpose(-1, -2)
+    p = torch.softmax(eager.logits(q, k, w["softmax_scale"], bias, w["causal"]).permute(0, 2, 1, 3), -1)
+    doh = do.permute(0, 2, 1, 3)
+    dp = doh @ v.permute(0, 2, 3, 1)
+    ds = p * (dp - (p * dp).sum(-1, keepdim=True))  # (B, H, Lq, Lk)
+    oh = ref[0].permute(0, 2, 1, 3)
+    var_delta = 2 * (u * u / 3) * ((oh * doh) ** 2).sum(-1, keepdim=True)  # o rounding, P rounding inside o
+    var_q = (u * u / 3) * ((ds ** 2) @ (kb ** 2)) + ((p @ kb) ** 2) * var_delta
+    var_k = (u * u / 3) * ((ds ** 2).transpose(-1, -2) @ (qb ** 2)) + (p ** 2).transpose(-1, -2) @ (qb ** 2 * var_delta)
+    for name, g, want, var, full in (("dq_bias", got[4], ref[5], var_q, w["q_bias"]),
+                                     ("dk_bias", got[5], ref[6], var_k, w["k_bias"])):
+        var = var.permute(0, 2, 1, 3)
+        dims = [i for i in (0, 2) if full.shape[i] == 1 and var.shape[i] != 1]
+        if dims:
+            var = var.sum(dim=dims, keepdim=True)
+        allowed = 6 * var.sqrt() + GRAD_TOL * want.abs().max()
+        assert ((g - want).abs() <= allowed).all(), (name, ((g - want).abs() / allowed).max())
+
+
+def test_workload_alibi(gpu_device):
+    """Causal ALiBi as an exact rank-2 bias, H=50 (reduced L).  o, dq, dk, dv pass the usual
+    gate; the two factor gradients pass the rounding-noise gate above."""
+    w = workloads.alibi(L=1024, H=50)
+    got, ref = _run_workload(gpu_device, w, torch.bfloat16, skip=("dq_bias", "dk_bias"))
+    _factor_grad_noise_gate(w, got, ref, torch.bfloat16)
+
+
+def test_workload_swin(gpu_device):
+    """Swin-V2 windows (reduced count), SVD factors shared by all windows; also reports how
+    close the rank-16 factors are to the exact table."""
+    w = workloads.swin(windows=8)
+    got, _ = _run_workload(gpu_device, w, torch.bfloat16)
+    assert w["bias_rel_error"].max() < 0.05
+    from oracle import eager
+    exact = eager.attention_eager(w["q"].float(), w["k"].float(), w["v"].float(), w["softmax_scale"],
+                                  w["bias_table"][None].expand(8, -1, -1, -1))
+    assert (got[0] - exact).abs().max() < 0.1
+
+
+def test_workload_pde(gpu_device):
+    """Exact rank-5 spatial-distance bias (reduced N); bias magnitudes up to ~30."""
+    _run_workload(gpu_device, workloads.pde(N=2048), torch.bfloat16)
+
+
+def test_workload_pairformer(gpu_device):
+    """Pairformer-shaped: rows as batch, rank-32 factors shared over rows (reduced N)."""
+    _run_workload(gpu_device, workloads.pairformer(N=192), torch.bfloat16)
+
+
+# ---------------------------------------------------------------- headline size: properties
+@pytest.fixture(scope="module")
+def headline(gpu_device):
+    w = workloads.sweep(workloads.HEADLINE["L"])
+    dev = gpu_device
+    t = {n: w[n].to(dev) for n in ("q", "k", "v", "q_bias", "k_bias", "do")}
+    leaves = [t[n].requires_grad_(True) for n in ("q", "k", "v", "q_bias", "k_bias")]
+    o = flash_bias_func(*leaves, None, False, w["softmax_scale"])
+    grads = torch.autograd.grad(o, leaves, t["do"])
+    torch.cuda.synchronize()
+    return w, t, o.detach(), grads
+
+
+def test_headline_rows_against_oracle(gpu_device, headline):
+    """At B2 H4 L16384 d32 r8 a query row depends on all keys but on no other query: o, dq,
+    dq_bias of a subset of rows are checked against the oracle run on (those rows, all keys)."""
+    w, t, o, grads = headline
+    rows = torch.cat([torch.arange(0, 64), torch.arange(8000, 8064), torch.arange(16320, 16384)])
+    sub = lambda x: x[:, rows]
+    ref = oracle(sub(w["q"]), w["k"], w["v"], sub(w["q_bias"]), w["k_bias"], None, False, w["softmax_scale"],
+                 sub(w["do"]))
+    err, _ = errors(o[:, rows].float().cpu(), ref[0])
+    assert err <= O_TOL[torch.bfloat16]
+    for got, want in ((grads[0], ref[2]), (grads[3], ref[5])):
+        _, rel = errors(got[:, rows].float().cpu(), want)
+        assert rel <= GRAD_TOL
+
+
+def test_headline_checksums(gpu_device, headline):
+    """Size-independent identities: rows of P sum to 1, so sum_j dv_j = sum_i dO_i; rows of dS
+    sum to 0, so sum_j dk_j = 0 and sum_j dk_bias_j = 0 (up to the rounding of the stored
+    gradients)."""
+    w, t, o, grads = headline
+    dv_sum = grads[2].float().sum(1)
+    do_sum = t["do"].float().sum(1)
+    assert (dv_sum - do_sum).abs().max() <= 0.02 * do_sum.abs().max()
+    for gk in (grads[1], grads[4]):
+        # every stored element, and every dS that went into it, carries a rounding error of 2^-9
+        bound = 16 * 2.0 ** -9 * gk.float().abs().sum(1).max() / math.sqrt(gk.shape[1])
+        assert gk.float().sum(1).abs().max() <= bound
+
+
+def test_headline_ones_value(gpu_device, headline):
+    w, t, _, _ = headline
+    o = flash_bias_func(t["q"], t["k"], torch.ones_like(t["v"]), t["q_bias"], t["k_bias"], None, False, None)
+    assert (o.float() - 1).abs().max() <= 2.0 ** -7
+
+
+def test_headline_matches_concat_sdpa(gpu_device, headline):
+    """Library cross-check at full size: the concat identity of
+    flash_bias/attention_func.py:188-237 evaluated by torch's fused attention on the GPU."""
+    w, t, o, grads = headline
+    q, k, v, qb, kb = [t[n].detach().requires_grad_(True) for n in ("q", "k", "v", "q_bias", "k_bias")]
+    s = w["softmax_scale"]
+    qc = torch.cat([q * s, qb], -1).transpose(1, 2)
+    kc = torch.cat([k, kb], -1).transpose(1, 2)
+    ref = torch.nn.functional.scaled_dot_product_attention(qc, kc, v.transpose(1, 2), scale=1.0).transpose(1, 2)
+    rgrads = torch.autograd.grad(ref, [q, k, v, qb, kb], t["do"])
+    assert (o.float() - ref.float()).abs().max() <= O_TOL[torch.bfloat16]
+    for got, want in zip(grads, rgrads):
+        _, rel = errors(got.float(), want.float())
+        assert rel <= GRAD_TOL
