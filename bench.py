@@ -1,0 +1,215 @@
+#!/usr/bin/env python3
+"""Benchmark of the FlashBias hot path on one MI355X.
+
+A step is one forward + backward of ``flash_bias_func`` on the headline workload of the
+reference's benchmark (flash_bias/config.py:12, flash_bias/benchmark.py:218-374): B2 H4 L16384
+d32 r8, non-causal, bf16, synthetic seeded inputs already resident in HBM.  Prints ONE JSON
+line:
+
+  value        whole-step throughput in TFLOP/s, algorithmic FLOPs 2 B H L^2 (7d + 4r)
+  ms_per_step  forward + backward wall time per step
+  roofline     the dominant kernel (backward main) timed alone with events on its stream,
+               against the dense bf16 MFMA peak
+  cpu_baseline the eager oracle (restated reference eager attention) on the host cores, on a
+               bounded sample of the same workload
+
+``--report`` instead prints a table over the other named workloads (not part of the contract).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
+PEAK_HBM_GBS = 8000.0
+
+
+def _to_dev(w, dev):
+    import torch
+    return {n: (t.to(dev) if isinstance(t, torch.Tensor) else t) for n, t in w.items()}
+
+
+def _time_events(fn, steps, warmup):
+    """Average milliseconds of fn() measured with events on the current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def _phase_timers(w, dev):
+    """Callables that launch the forward and the three backward phases alone through the C
+    ABI (buffers allocated once, outside the timed region)."""
+    import torch
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _prepare, _stream, _tensor
+    lib = _lib.load()
+    q, k, v, qb, kb, do = (w[n] for n in ("q", "k", "v", "q_bias", "k_bias", "do"))
+    p, keep = _prepare(q, k, v, qb, kb, None, w["causal"], w["softmax_scale"])
+    o = torch.empty_like(q)
+    lse = torch.empty((p.B, p.H, p.Lq), device=dev, dtype=torch.float32)
+    p.o, p.lse = _tensor(o), lse.data_ptr()
+    grads = [torch.empty_like(t) for t in (q, k, v)]
+    p.dout, p.dq, p.dk, p.dv = _tensor(do), _tensor(grads[0]), _tensor(grads[1]), _tensor(grads[2])
+    if qb is not None:
+        full = [torch.empty((p.B, L, p.H, p.r), device=dev, dtype=q.dtype) for L in (p.Lq, p.Lk)]
+        p.dq_bias, p.dk_bias = _tensor(full[0]), _tensor(full[1])
+        keep += full
+    delta = torch.empty_like(lse)
+    nbytes = lib.fb_bwd_workspace_bytes(p)
+    ws = torch.empty(nbytes // 4, device=dev, dtype=torch.float32)
+    p.delta, p.workspace, p.workspace_bytes = delta.data_ptr(), ws.data_ptr(), nbytes
+    keep += [o, lse, grads, delta, ws]
+
+    def call(fn):
+        def run():
+            _lib.check_status(fn(p, _stream()))
+        return run
+    return {name: call(getattr(lib, name)) for name in
+            ("fb_fwd", "fb_bwd_preprocess", "fb_bwd_main", "fb_bwd_finalize")}, keep
+
+
+def _cpu_baseline(w, flops_per_slice):
+    """Eager oracle, fp32, all host cores, on ONE (batch, head) slice of the workload at full
+    sequence length (the (L, L) fp32 intermediates are 1 GiB each at L=16384)."""
+    import torch
+    from oracle import eager
+    cores = os.cpu_count() or 1
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        pass
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    sl = lambda t: t[:1, :, :1].float().cpu()
+    args = (sl(w["q"]), sl(w["k"]), sl(w["v"]), sl(w["q_bias"]), sl(w["k_bias"]), None, w["causal"],
+            w["softmax_scale"])
+    t0 = time.perf_counter()
+    eager.flashbias_eager_grads(*args, sl(w["do"]))
+    dt = time.perf_counter() - t0
+    return {"value": round(flops_per_slice / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "seconds": round(dt, 2),
+            "sample": "1 of B*H (batch, head) slices at full L, one fwd+bwd of the eager oracle in fp32"}
+
+
+def headline(args):
+    import torch
+    from flashbias_amd import flash_bias_func, workloads
+    dev = torch.device("cuda:0")
+    hl = workloads.HEADLINE
+    w = _to_dev(workloads.sweep(hl["L"], hl["B"], hl["H"], hl["d"], hl["r"], torch.bfloat16, seed=0), dev)
+    leaves = [w[n].requires_grad_(True) for n in ("q", "k", "v", "q_bias", "k_bias")]
+
+    def step():
+        o = flash_bias_func(*leaves, None, False, w["softmax_scale"])
+        return torch.autograd.grad(o, leaves, w["do"])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    f_fwd, f_bwd = workloads.flops(hl["B"], hl["H"], hl["L"], hl["L"], hl["d"], hl["r"])
+    phases, keep = _phase_timers({n: (t.detach() if isinstance(t, torch.Tensor) else t) for n, t in w.items()}, dev)
+    ms = {name: _time_events(fn, args.steps, max(1, args.warmup)) for name, fn in phases.items()}
+    # the backward main kernel: everything of the backward except delta (2 B H L d) and the casts
+    f_main = f_bwd
+    tflops_main = f_main / (ms["fb_bwd_main"] * 1e-3) / 1e12
+    value = (f_fwd + f_bwd) / (ms_step * 1e-3) / 1e12
+    ref_fwd, ref_fb = workloads.reference_formula_flops(hl["B"], hl["H"], hl["L"], hl["d"])
+    out = {
+        "metric": "fwd+bwd ms & TFLOP/s (% bf16 MFMA peak) at B2 H4 L16384 d32 r8, 1 GPU",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "flash_bias_func fwd+bwd, B2 H4 L16384 d32 r8, non-causal, bf16 "
+                               "(flash_bias/config.py:12 at len=16384)"},
+        "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
+        "fwd_ms": round(ms["fb_fwd"], 4),
+        "fwd_tflops": round(f_fwd / (ms["fb_fwd"] * 1e-3) / 1e12, 2),
+        "bwd_ms": round(ms["fb_bwd_preprocess"] + ms["fb_bwd_main"] + ms["fb_bwd_finalize"], 4),
+        "kernel_ms": {k: round(v, 4) for k, v in ms.items()},
+        "reference_formula_tflops": round(ref_fb / (ms_step * 1e-3) / 1e12, 2),
+        "roofline": {"kernel": "bwd_kernel (fb_bwd_main)", "bound": "mfma", "achieved": round(tflops_main, 2),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_main / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None},
+    }
+    del keep
+    if not args.no_cpu:
+        out["cpu_baseline"] = _cpu_baseline(w, (f_fwd + f_bwd) / (hl["B"] * hl["H"]))
+    print(json.dumps(out))
+
+
+def report(args):
+    """fwd / fwd+bwd milliseconds and TFLOP/s over the named workloads (informational)."""
+    import torch
+    from flashbias_amd import workloads
+    dev = torch.device("cuda:0")
+    rows = []
+    cases = [(f"sweep L={L}", lambda L=L: workloads.sweep(L)) for L in workloads.SWEEP_LENGTHS]
+    cases += [(f"alibi causal L={L}", lambda L=L: workloads.alibi(L)) for L in (2048, 4096, 8192)]
+    cases += [("swin 4096x256 r16", lambda: workloads.swin()), ("pde N=32768 r5", lambda: workloads.pde()),
+              ("pairformer 768 r32", lambda: workloads.pairformer())]
+    for name, make in cases:
+        w = _to_dev(make(), dev)
+        B, Lq, H, d = w["q"].shape
+        r = w["q_bias"].shape[-1]
+        f_fwd, f_bwd = workloads.flops(B, H, Lq, w["k"].shape[1], d, r, w["causal"])
+        phases, keep = _phase_timers(w, dev)
+        ms = {n: _time_events(fn, args.steps, args.warmup) for n, fn in phases.items()}
+        bwd = ms["fb_bwd_preprocess"] + ms["fb_bwd_main"] + ms["fb_bwd_finalize"]
+        rows.append((name, ms["fb_fwd"], f_fwd / ms["fb_fwd"] / 1e9, ms["fb_fwd"] + bwd,
+                     (f_fwd + f_bwd) / (ms["fb_fwd"] + bwd) / 1e9))
+        del keep, w
+        torch.cuda.empty_cache()
+    print("| workload | fwd ms | fwd TFLOP/s | fwd+bwd ms | fwd+bwd TFLOP/s | % bf16 peak |")
+    print("|---|---|---|---|---|---|")
+    for name, a, b, c, d_ in rows:
+        print(f"| {name} | {a:.3f} | {b:.1f} | {c:.3f} | {d_:.1f} | {100 * d_ / PEAK_BF16_TFLOPS:.1f} |")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--report", action="store_true", help="table over all named workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the path has no collective; (batch, head) pairs are "
+                 "independent and would be split across GPUs with no exchange. Run with --gpus 1.")
+    from flashbias_amd import _lib
+    _lib.load()  # fail loudly if the HIP library is not built
+    if args.report:
+        report(args)
+    else:
+        headline(args)
+
+
+if __name__ == "__main__":
+    main()
