@@ -26,9 +26,11 @@
 namespace fb {
 
 // ------------------------------------------------------------------------------------ main
-template <class T, int NKD_, int NKR_, int NDV_>
+// VEC: every streamed tensor is 16-byte aligned (base and strides) and d, r are multiples of 8.
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_>
 struct BwdCfg {
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
+    static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int BN = 32 * NWAVES; // keys per workgroup
     static constexpr int QBLK = 2, BMQ = 32 * QBLK; // queries per step
@@ -89,16 +91,13 @@ __device__ __forceinline__ void bwd_load_step(BwdStage<C> &st, const BwdArgs &a,
         bwd_task<C>(task, kind, quad, ch);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            st.x[i][j] = u32x4_t{0u, 0u, 0u, 0u};
             const int query = m0 + quad * 4 + j;
-            if (task < C::TASKS && query < a.Lq) {
-                if (kind == 0)
-                    st.x[i][j] = load_chunk(qbase + (int64_t)query * a.q.ss, ch * 8, a.d, a.q.vec_ok);
-                else if (kind == 1)
-                    st.x[i][j] = load_chunk(qbbase + (int64_t)query * a.qb.ss, ch * 8, a.r, a.qb.vec_ok);
-                else
-                    st.x[i][j] = load_chunk(dobase + (int64_t)query * a.dout.ss, ch * 8, a.d, a.dout.vec_ok);
-            }
+            // one load per task: pick the tensor by lane (all three share the chunk geometry)
+            const uint16_t *base = kind == 0 ? qbase : kind == 1 ? qbbase : dobase;
+            const int64_t ld = kind == 0 ? a.q.ss : kind == 1 ? a.qb.ss : a.dout.ss;
+            const int ncols = kind == 1 ? a.r : a.d;
+            st.x[i][j] = u32x4_t{0u, 0u, 0u, 0u};
+            if (task < C::TASKS) st.x[i][j] = load_chunk<C::VEC>(base, ld, query, a.Lq, ch * 8, ncols);
         }
     }
     st.lse2 = INFINITY; // rows past the end: P = exp2(-inf) = 0
@@ -184,7 +183,7 @@ __global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
     const float *lse = a.lse + (int64_t)bh * a.Lq;
     const float *delta = a.delta + (int64_t)bh * a.Lq;
     const uint8_t *mbase = nullptr;
-    if (a.mask.type)
+    if constexpr (C::MASK)
         mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
@@ -193,18 +192,14 @@ __global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
     u32x4_t vreg[C::NKD]; // B operand of dP
 #pragma unroll
     for (int t = 0; t < C::NK; ++t) {
-        kreg[t] = u32x4_t{0u, 0u, 0u, 0u};
-        if (key < a.Lk) {
-            if (t < C::NKD)
-                kreg[t] = load_chunk(kbase + (int64_t)key * a.k.ss, 16 * t + 8 * g, a.d, a.k.vec_ok);
-            else if constexpr (C::NKR > 0)
-                kreg[t] = load_chunk(kbbase + (int64_t)key * a.kb.ss, 16 * (t - C::NKD) + 8 * g, a.r, a.kb.vec_ok);
-        }
+        if (t < C::NKD)
+            kreg[t] = load_chunk<C::VEC>(kbase, a.k.ss, key, a.Lk, 16 * t + 8 * g, a.d);
+        else if constexpr (C::NKR > 0)
+            kreg[t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, 16 * (t - C::NKD) + 8 * g, a.r);
     }
 #pragma unroll
     for (int t = 0; t < C::NKD; ++t) {
-        vreg[t] = u32x4_t{0u, 0u, 0u, 0u};
-        if (key < a.Lk) vreg[t] = load_chunk(vbase + (int64_t)key * a.v.ss, 16 * t + 8 * g, a.d, a.v.vec_ok);
+        vreg[t] = load_chunk<C::VEC>(vbase, a.v.ss, key, a.Lk, 16 * t + 8 * g, a.d);
     }
     // A operand of phase 2: rows = channels of [K|K_b] (32 per block), k-slots = the 128 keys
     // of the workgroup in natural order.
@@ -298,7 +293,7 @@ __global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
                 for (int t = 0; t < C::NKD; ++t)
                     dp = T::mfma(*reinterpret_cast<const u32x4_t *>(sdO + (qb * 32 + c) * C::DOP + 16 * t + 8 * g),
                                  vreg[t], dp);
-                if (a.mask.type) {
+                if constexpr (C::MASK) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
                         s[v] += mask_at_b<T>(a.mask, mbase, m0 + qb * 32 + 8 * (v >> 2) + 4 * g + (v & 3), key, a.Lq,
@@ -420,9 +415,9 @@ __global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
 }
 
 // ------------------------------------------------------------------------------- launchers
-template <class T, int NKD, int NKR, int NDV>
-static hipError_t launch_bwd_cfg(const BwdArgs &a0, hipStream_t stream) {
-    typedef BwdCfg<T, NKD, NKR, NDV> C;
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+static hipError_t launch_bwd_vec(const BwdArgs &a0, hipStream_t stream) {
+    typedef BwdCfg<T, NKD, NKR, NDV, VEC, MASK> C;
     BwdArgs a = a0;
     a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
     auto kern = bwd_kernel<T, C>;
@@ -434,6 +429,17 @@ static hipError_t launch_bwd_cfg(const BwdArgs &a0, hipStream_t stream) {
     const int total = a.ntiles_n * a.B * a.H;
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
+}
+
+template <class T, int NKD, int NKR, int NDV>
+static hipError_t launch_bwd_cfg(const BwdArgs &a, hipStream_t stream) {
+    const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+    if (a.mask.type)
+        return vec ? launch_bwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
+                   : launch_bwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    return vec ? launch_bwd_vec<T, NKD, NKR, NDV, true, false>(a, stream)
+               : launch_bwd_vec<T, NKD, NKR, NDV, false, false>(a, stream);
 }
 
 template <class T, int NKD, int NDV>

@@ -16,9 +16,16 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a, in
         const uint16_t *orow = a.o.ptr + b * a.o.sb + h * a.o.sh + (int64_t)i * a.o.ss;
         const uint16_t *drow = a.dout.ptr + b * a.dout.sb + h * a.dout.sh + (int64_t)i * a.dout.ss;
         float acc = 0.f;
+        const bool vec = a.o.vec_ok && a.dout.vec_ok && a.d % 8 == 0;
         for (int c0 = 0; c0 < a.d; c0 += 8) {
-            const u32x4_t x = load_chunk(orow, c0, a.d, a.o.vec_ok);
-            const u32x4_t y = load_chunk(drow, c0, a.d, a.dout.vec_ok);
+            u32x4_t x, y;
+            if (vec) {
+                x = load_chunk<true>(orow, 0, 0, 1, c0, a.d);
+                y = load_chunk<true>(drow, 0, 0, 1, c0, a.d);
+            } else {
+                x = load_chunk<false>(orow, 0, 0, 1, c0, a.d);
+                y = load_chunk<false>(drow, 0, 0, 1, c0, a.d);
+            }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 acc += T::to_float((uint16_t)(x[e] & 0xffffu)) * T::to_float((uint16_t)(y[e] & 0xffffu));

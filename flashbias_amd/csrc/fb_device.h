@@ -82,17 +82,32 @@ struct MaskDesc {
     int is_f32; // else same 16-bit type as the inputs
 };
 
-// Eight consecutive channels [col0, col0 + 8) of one row; zero beyond ncols.
-__device__ __forceinline__ u32x4_t load_chunk(const uint16_t *row, int col0, int ncols, bool vec_ok) {
-    u32x4_t out = {0u, 0u, 0u, 0u};
-    if (col0 + 8 <= ncols && vec_ok) {
-        out = *reinterpret_cast<const u32x4_t *>(row + col0);
-    } else if (col0 < ncols) {
-        uint16_t e[8];
+// Eight consecutive channels [col0, col0 + 8) of row `row` of a (rows x ncols) matrix with row
+// stride `ld`; zero beyond ncols and for row >= nrows.  Branch-free: out-of-range lanes read a
+// clamped (valid) address and the result is zeroed by a select.  VEC = one 16-byte load
+// (requires 16-byte aligned base / strides and ncols % 8 == 0), else eight 2-byte loads.
+template <bool VEC>
+__device__ __forceinline__ u32x4_t load_chunk(const uint16_t *base, int64_t ld, int row, int nrows, int col0,
+                                              int ncols) {
+    const bool row_ok = row < nrows;
+    const uint16_t *rp = base + (int64_t)(row_ok ? row : nrows - 1) * ld;
+    u32x4_t out;
+    if constexpr (VEC) {
+        const bool ok = row_ok && col0 < ncols;
+        out = *reinterpret_cast<const u32x4_t *>(rp + (col0 < ncols ? col0 : 0));
 #pragma unroll
-        for (int i = 0; i < 8; ++i) e[i] = (col0 + i < ncols) ? row[col0 + i] : (uint16_t)0;
+        for (int i = 0; i < 4; ++i) out[i] = ok ? out[i] : 0u;
+    } else {
+        uint32_t e[8];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = (uint32_t)e[2 * i] | ((uint32_t)e[2 * i + 1] << 16);
+        for (int i = 0; i < 8; ++i) {
+            const int col = col0 + i;
+            uint32_t val = rp[col < ncols ? col : ncols - 1];
+            asm volatile("" : "+v"(val)); // keep the load unconditional (no per-lane branch)
+            e[i] = (row_ok && col < ncols) ? val : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = e[2 * i] | (e[2 * i + 1] << 16);
     }
     return out;
 }

@@ -19,9 +19,11 @@
 
 namespace fb {
 
-template <class T, int NKD_, int NKR_, int NDV_, int QBLK_>
+// VEC: every streamed tensor is 16-byte aligned (base and strides) and d, r are multiples of 8.
+template <class T, int NKD_, int NKR_, int NDV_, int QBLK_, bool VEC_, bool MASK_>
 struct FwdCfg {
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_, QBLK = QBLK_;
+    static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int BM = NWAVES * QBLK * 32;
     static constexpr int KBLK = 2, BN = 32 * KBLK;
@@ -53,18 +55,16 @@ __device__ __forceinline__ void fwd_load_tile(FwdStage<C> &st, const FwdArgs &a,
     for (int i = 0; i < C::K_PT; ++i) {
         const int task = tid + i * C::NTHREADS;
         const int row = task / C::CD, ch = task % C::CD;
-        st.k[i] = u32x4_t{0u, 0u, 0u, 0u};
-        if (task < C::K_TASKS && n0 + row < a.Lk)
-            st.k[i] = load_chunk(kbase + (int64_t)(n0 + row) * a.k.ss, ch * 8, a.d, a.k.vec_ok);
+        if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS)
+            st.k[i] = load_chunk<C::VEC>(kbase, a.k.ss, n0 + row, a.Lk, ch * 8, a.d);
     }
     if constexpr (C::NKR > 0) {
 #pragma unroll
         for (int i = 0; i < C::KB_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
             const int row = task / C::CR, ch = task % C::CR;
-            st.kb[i] = u32x4_t{0u, 0u, 0u, 0u};
-            if (task < C::KB_TASKS && n0 + row < a.Lk)
-                st.kb[i] = load_chunk(kbbase + (int64_t)(n0 + row) * a.kb.ss, ch * 8, a.r, a.kb.vec_ok);
+            if (C::KB_TASKS % C::NTHREADS == 0 || task < C::KB_TASKS)
+                st.kb[i] = load_chunk<C::VEC>(kbbase, a.kb.ss, n0 + row, a.Lk, ch * 8, a.r);
         }
     }
 #pragma unroll
@@ -73,10 +73,8 @@ __device__ __forceinline__ void fwd_load_tile(FwdStage<C> &st, const FwdArgs &a,
         const int quad = task / (C::DV / 8), ch = task % (C::DV / 8);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            st.v[i][j] = u32x4_t{0u, 0u, 0u, 0u};
-            const int key = n0 + quad * 4 + j;
-            if (task < C::V_TASKS && key < a.Lk)
-                st.v[i][j] = load_chunk(vbase + (int64_t)key * a.v.ss, ch * 8, a.d, a.v.vec_ok);
+            if (C::V_TASKS % C::NTHREADS == 0 || task < C::V_TASKS)
+                st.v[i][j] = load_chunk<C::VEC>(vbase, a.v.ss, n0 + quad * 4 + j, a.Lk, ch * 8, a.d);
         }
     }
 }
@@ -126,7 +124,7 @@ __device__ __forceinline__ float mask_at(const MaskDesc &m, const uint8_t *base,
 }
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) void fwd_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 3))) void fwd_kernel(const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *sKbuf = reinterpret_cast<uint16_t *>(smem);
     uint16_t *sVbuf = sKbuf + 2 * C::SK_ELEMS;
@@ -152,7 +150,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_kernel(const FwdArgs a) {
         kbbase = a.kb.ptr + b * a.kb.sb + h * a.kb.sh;
     }
     const uint8_t *mbase = nullptr;
-    if (a.mask.type)
+    if constexpr (C::MASK)
         mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
@@ -163,14 +161,10 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_kernel(const FwdArgs a) {
         const int query = wq0 + qb * 32 + c;
 #pragma unroll
         for (int t = 0; t < C::NK; ++t) {
-            qreg[qb][t] = u32x4_t{0u, 0u, 0u, 0u};
-            if (query < a.Lq) {
-                if (t < C::NKD)
-                    qreg[qb][t] = load_chunk(qbase + (int64_t)query * a.q.ss, 16 * t + 8 * g, a.d, a.q.vec_ok);
-                else if constexpr (C::NKR > 0)
-                    qreg[qb][t] = load_chunk(qbbase + (int64_t)query * a.qb.ss, 16 * (t - C::NKD) + 8 * g, a.r,
-                                             a.qb.vec_ok);
-            }
+            if (t < C::NKD)
+                qreg[qb][t] = load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d);
+            else if constexpr (C::NKR > 0)
+                qreg[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * (t - C::NKD) + 8 * g, a.r);
         }
     }
 
@@ -230,7 +224,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_kernel(const FwdArgs a) {
                 }
             }
             // ---- additive mask, then -inf for keys past the end and causal-hidden pairs
-            if (a.mask.type) {
+            if constexpr (C::MASK) {
 #pragma unroll
                 for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
@@ -322,7 +316,7 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_kernel(const FwdArgs a) {
 #pragma unroll
                 for (int bq = 0; bq < 4; ++bq) {
                     const int ch = 32 * n + 8 * bq + 4 * g;
-                    if (ch + 4 <= a.d && a.o.vec_ok) {
+                    if (C::VEC && ch + 4 <= a.d) {
                         u32x2_t pk;
                         pk[0] = T::pack2(acc_o[qb][n][4 * bq] * inv, acc_o[qb][n][4 * bq + 1] * inv);
                         pk[1] = T::pack2(acc_o[qb][n][4 * bq + 2] * inv, acc_o[qb][n][4 * bq + 3] * inv);
@@ -337,10 +331,10 @@ __global__ __launch_bounds__(C::NTHREADS) void fwd_kernel(const FwdArgs a) {
     }
 }
 
-template <class T, int NKD, int NKR, int NDV>
-static hipError_t launch_fwd_cfg(const FwdArgs &a0, hipStream_t stream) {
-    constexpr int QBLK = (NKD + NKR <= 4 && NDV <= 2) ? 2 : 1;
-    typedef FwdCfg<T, NKD, NKR, NDV, QBLK> C;
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+static hipError_t launch_fwd_vec(const FwdArgs &a0, hipStream_t stream) {
+    constexpr int QBLK = 1;
+    typedef FwdCfg<T, NKD, NKR, NDV, QBLK, VEC, MASK> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_kernel<T, C>;
@@ -352,6 +346,17 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a0, hipStream_t stream) {
     const int total = a.ntiles_m * a.B * a.H;
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
+}
+
+template <class T, int NKD, int NKR, int NDV>
+static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
+    const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.o.vec_ok && a.d % 8 == 0 &&
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+    if (a.mask.type)
+        return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
+                   : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, false>(a, stream)
+               : launch_fwd_vec<T, NKD, NKR, NDV, false, false>(a, stream);
 }
 
 template <class T, int NKD, int NDV>
