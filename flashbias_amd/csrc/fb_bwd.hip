@@ -55,6 +55,9 @@ struct BwdCfg {
     static constexpr int QUADS = BMQ / 4;
     static constexpr int TASKS = QUADS * (CQ + CR + CO);
     static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
+    // register budget: 2 waves per SIMD (256 registers each) for the small shapes, which keeps
+    // the MFMA accumulators in ordinary VGPRs; the big ones need the whole file
+    static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 2 : 1;
 };
 
 template <class C>
@@ -154,7 +157,7 @@ __device__ __forceinline__ float mask_at_b(const MaskDesc &m, const uint8_t *bas
 }
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU))) void bwd_kernel(const BwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
     uint16_t *sdS = stage0 + C::STAGE_ELEMS;
@@ -242,17 +245,26 @@ __global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
     const int step0 = a.causal ? n0 / C::BMQ : 0;
     const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
 
+    // Workgroups of one (batch, head) walk the query steps in rotated order: at any moment
+    // they add into different rows of the dq workspace instead of all hitting the same ones.
+    const int span = nsteps - step0;
+    const int rot = span > 0 ? (int)(((int64_t)tile_n * 7) % span) : 0;
+    auto step_of = [&](int it) {
+        const int x = it + rot;
+        return step0 + (x >= span ? x - span : x);
+    };
+
     BwdStage<C> st;
-    if (step0 < nsteps) {
-        bwd_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, step0 * C::BMQ, tid);
+    if (span > 0) {
+        bwd_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, step_of(0) * C::BMQ, tid);
         bwd_store_step<C>(st, stage0, tid);
     }
     __syncthreads();
 
-    for (int step = step0; step < nsteps; ++step) {
-        const int m0 = step * C::BMQ;
-        const bool more = step + 1 < nsteps;
-        if (more) bwd_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, m0 + C::BMQ, tid);
+    for (int it = 0; it < span; ++it) {
+        const int m0 = step_of(it) * C::BMQ;
+        const bool more = it + 1 < span;
+        if (more) bwd_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, step_of(it + 1) * C::BMQ, tid);
 
         const uint16_t *sQ = stage0;
         const uint16_t *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
@@ -364,7 +376,11 @@ __global__ __launch_bounds__(C::NTHREADS) void bwd_kernel(const BwdArgs a) {
                     } else if (ch - 16 * C::NKD < a.r) {
                         row = a.r_row0 + ch - 16 * C::NKD;
                     }
+#ifdef FB_EXPERIMENT_NO_ATOMIC
+                    if (row >= 0 && acc[v] == 12345.678f) dq_bh[(int64_t)row * a.lq_pad + query] = acc[v];
+#else
                     if (row >= 0) unsafeAtomicAdd(dq_bh + (int64_t)row * a.lq_pad + query, acc[v]);
+#endif
                 }
             }
         };
