@@ -1,31 +1,41 @@
 // Forward FlashBias attention for gfx950:  o = softmax(scale q k^T + q_b k_b^T + mask) v, lse.
 // Replaces _fwd_kernel of the reference (flash_bias/flash_bias_triton.py:62-355).
 //
-// One workgroup (4 waves) owns BM = 128 * QBLK consecutive queries of one (batch, head); each
-// wave owns 32 * QBLK of them.  Keys are streamed in tiles of BN = 64 through double-buffered
-// LDS.  Everything is computed transposed so that a lane owns one query:
+// One workgroup (4 waves) owns BM = 128 consecutive queries of one (batch, head); each wave
+// owns 32 of them.  Keys are streamed in tiles of BN = 64 through double-buffered LDS.
+// Everything is computed transposed so that a lane owns one query:
 //
-//   S^T (keys x queries) = [K | K_b] [Q | Q_b]^T       A = key tile from LDS, B = query regs
-//   O^T (d x queries)   += V^T P^T                     A = V^T tile from LDS, B = P^T regs
+//   S^T (keys x queries) = [K | K_b] [scale Q | Q_b]^T     A = key tile from LDS, B = query regs
+//   O^T (d x queries)   += V^T P^T                         A = V^T tile from LDS, B = P^T regs
 //
-// In the C layout a lane holds one query column and 16 keys of it, so the row max / sum of
-// the online softmax are in-lane reductions plus one exchange with lane ^ 32, the rescale
-// factor is a per-lane scalar, and P^T is already in the B-operand layout of the second MFMA
-// (no LDS round trip for P).  The contraction runs over the concatenated channels
-// [d | r], zero-padded in LDS to 16-wide MFMA steps; the fp32 accumulator is multiplied by
-// the softmax scale after the d steps and before the r steps, so the bias product is never
-// scaled (flash_bias_triton.py:246-256).
+// In the C layout a lane holds one query column and 16 keys of it, so the row max of the
+// online softmax is an in-lane reduction plus one exchange with lane ^ 32, the rescale factor
+// is a per-lane scalar, and P^T is already in the B-operand layout of the second MFMA (no LDS
+// round trip for P).  The contraction runs over the concatenated channels [d | r],
+// zero-padded to 16-wide MFMA steps.
+//
+// Softmax scale: the reference multiplies the fp32 q k^T accumulator by the scale and never
+// scales the bias product (flash_bias_triton.py:246-256).  Here scale * q is formed in fp32 when
+// the query operand is loaded and split into two 16-bit parts hi + lo (hi = round(x),
+// lo = round(x - hi)), both contracted against the same key registers: the product carries 16
+// mantissa bits of scale * q, the bias factors stay untouched, and the inner loop needs no
+// multiply per score.
+//
+// The VALU, not the MFMA pipe, bounds this kernel at d = 32, so the per-score work is kept to:
+// max3, fma + exp2, convert, and a 2-way dot for the row sum; the running reference of the
+// softmax only moves when a row maximum grows by more than 2^8 (then p <= 256, exact enough in
+// fp32 / 16-bit), so the accumulator rescale is rare.
 #include "fb_kernels.h"
 
 namespace fb {
 
 // VEC: every streamed tensor is 16-byte aligned (base and strides) and d, r are multiples of 8.
-template <class T, int NKD_, int NKR_, int NDV_, int QBLK_, bool VEC_, bool MASK_>
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_>
 struct FwdCfg {
-    static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_, QBLK = QBLK_;
+    static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
-    static constexpr int BM = NWAVES * QBLK * 32;
+    static constexpr int BM = NWAVES * 32;
     static constexpr int KBLK = 2, BN = 32 * KBLK;
     static constexpr int NK = NKD + NKR;
     static constexpr int DKP = 16 * NK + 8; // LDS row of [K | K_b], elements (16 B of padding)
@@ -33,86 +43,154 @@ struct FwdCfg {
     static constexpr int BNP = BN + 8; // LDS row of V^T
     static constexpr int SK_ELEMS = BN * DKP, SV_ELEMS = DV * BNP;
     static constexpr int LDS_BYTES = 2 * (SK_ELEMS + SV_ELEMS) * 2;
-    // cooperative loader: 8-channel chunks of K and K_b, (4 keys x 8 channels) blocks of V
+    // cooperative loader: 8-channel chunks of K and K_b (one key row each), (4 keys x 4
+    // channels) blocks of V.  Consecutive threads take consecutive rows / key quads, which
+    // keeps the LDS writes free of bank conflicts.
     static constexpr int CD = 2 * NKD, CR = 2 * NKR;
-    static constexpr int K_TASKS = BN * CD, KB_TASKS = BN * CR, V_TASKS = (BN / 4) * (DV / 8);
+    static constexpr int K_TASKS = BN * CD, KB_TASKS = BN * CR, V_TASKS = (BN / 4) * (DV / 4);
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int KB_PT = (KB_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
+    static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 3 : 2;
 };
 
 template <class C>
 struct FwdStage { // one key tile in flight from HBM to LDS
     u32x4_t k[C::K_PT];
     u32x4_t kb[C::KB_PT > 0 ? C::KB_PT : 1];
-    u32x4_t v[C::V_PT][4];
+    u32x2_t v[C::V_PT][4];
 };
 
-template <class C>
-__device__ __forceinline__ void fwd_load_tile(FwdStage<C> &st, const FwdArgs &a, const uint16_t *kbase,
-                                              const uint16_t *kbbase, const uint16_t *vbase, int n0, int tid) {
+// Four consecutive channels [col0, col0 + 4) of one row, zero outside the matrix.
+template <bool VEC>
+__device__ __forceinline__ u32x2_t load_half(const uint16_t *base, int64_t ld, int row, int nrows, int col0,
+                                             int ncols) {
+    const bool row_ok = row < nrows;
+    const uint16_t *rp = base + (int64_t)(row_ok ? row : nrows - 1) * ld;
+    u32x2_t out;
+    if constexpr (VEC) {
+        const bool ok = row_ok && col0 < ncols;
+        out = *reinterpret_cast<const u32x2_t *>(rp + (col0 < ncols ? col0 : 0));
+        out[0] = ok ? out[0] : 0u;
+        out[1] = ok ? out[1] : 0u;
+    } else {
+        uint32_t e[4];
 #pragma unroll
-    for (int i = 0; i < C::K_PT; ++i) {
-        const int task = tid + i * C::NTHREADS;
-        const int row = task / C::CD, ch = task % C::CD;
-        if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS)
-            st.k[i] = load_chunk<C::VEC>(kbase, a.k.ss, n0 + row, a.Lk, ch * 8, a.d);
-    }
-    if constexpr (C::NKR > 0) {
-#pragma unroll
-        for (int i = 0; i < C::KB_PT; ++i) {
-            const int task = tid + i * C::NTHREADS;
-            const int row = task / C::CR, ch = task % C::CR;
-            if (C::KB_TASKS % C::NTHREADS == 0 || task < C::KB_TASKS)
-                st.kb[i] = load_chunk<C::VEC>(kbbase, a.kb.ss, n0 + row, a.Lk, ch * 8, a.r);
+        for (int i = 0; i < 4; ++i) {
+            const int col = col0 + i;
+            uint32_t val = rp[col < ncols ? col : ncols - 1];
+            asm volatile("" : "+v"(val));
+            e[i] = (row_ok && col < ncols) ? val : 0u;
         }
+        out[0] = e[0] | (e[1] << 16);
+        out[1] = e[2] | (e[3] << 16);
     }
-#pragma unroll
-    for (int i = 0; i < C::V_PT; ++i) {
-        const int task = (C::NTHREADS - 1 - tid) + i * C::NTHREADS;
-        const int quad = task / (C::DV / 8), ch = task % (C::DV / 8);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            if (C::V_TASKS % C::NTHREADS == 0 || task < C::V_TASKS)
-                st.v[i][j] = load_chunk<C::VEC>(vbase, a.v.ss, n0 + quad * 4 + j, a.Lk, ch * 8, a.d);
-        }
-    }
+    return out;
 }
 
+// Per-thread constants of the cooperative loader: which rows / chunks this thread copies, as
+// 32-bit element offsets from the (wave-uniform) base of a key tile, so that the per-tile
+// address is "scalar base + lane offset" and costs no vector ALU work.
 template <class C>
-__device__ __forceinline__ void fwd_store_tile(const FwdStage<C> &st, uint16_t *sK, uint16_t *sVt, int tid) {
+struct FwdLoader {
+    uint32_t koff[C::K_PT], kboff[C::KB_PT > 0 ? C::KB_PT : 1], voff[C::V_PT][4];
+    uint32_t kdst[C::K_PT], kbdst[C::KB_PT > 0 ? C::KB_PT : 1], vdst[C::V_PT];
+    bool kok[C::K_PT], kbok[C::KB_PT > 0 ? C::KB_PT : 1], vok[C::V_PT];
+
+    __device__ __forceinline__ void init(const FwdArgs &a, int tid) {
 #pragma unroll
-    for (int i = 0; i < C::K_PT; ++i) {
-        const int task = tid + i * C::NTHREADS;
-        const int row = task / C::CD, ch = task % C::CD;
-        if (task < C::K_TASKS) *reinterpret_cast<u32x4_t *>(sK + row * C::DKP + ch * 8) = st.k[i];
-    }
-    if constexpr (C::NKR > 0) {
+        for (int i = 0; i < C::K_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            const int row = task % C::BN, ch = task / C::BN;
+            kok[i] = task < C::K_TASKS && ch * 8 < a.d;
+            koff[i] = kok[i] ? (uint32_t)(row * a.k.ss + ch * 8) : 0u;
+            kdst[i] = row * C::DKP + ch * 8;
+        }
 #pragma unroll
         for (int i = 0; i < C::KB_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
-            const int row = task / C::CR, ch = task % C::CR;
-            if (task < C::KB_TASKS)
-                *reinterpret_cast<u32x4_t *>(sK + row * C::DKP + 16 * C::NKD + ch * 8) = st.kb[i];
+            const int row = task % C::BN, ch = task / C::BN;
+            kbok[i] = task < C::KB_TASKS && ch * 8 < a.r;
+            kboff[i] = kbok[i] ? (uint32_t)(row * a.kb.ss + ch * 8) : 0u;
+            kbdst[i] = row * C::DKP + 16 * C::NKD + ch * 8;
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) {
+            const int task = (C::NTHREADS - 1 - tid) + i * C::NTHREADS;
+            const int quad = task % (C::BN / 4), hc = task / (C::BN / 4);
+            vok[i] = task < C::V_TASKS && hc * 4 < a.d;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) voff[i][j] = vok[i] ? (uint32_t)((quad * 4 + j) * a.v.ss + hc * 4) : 0u;
+            vdst[i] = (hc * 4) * C::BNP + slot_of(quad * 4); // 4 keys stay adjacent, quads are permuted
         }
     }
+
+    // Tile fully inside the sequence, 16-byte aligned tensors: plain loads, nothing else.
+    __device__ __forceinline__ void load_fast(FwdStage<C> &st, const uint16_t *kt, const uint16_t *kbt,
+                                              const uint16_t *vt) const {
 #pragma unroll
-    for (int i = 0; i < C::V_PT; ++i) {
-        const int task = (C::NTHREADS - 1 - tid) + i * C::NTHREADS;
-        const int quad = task / (C::DV / 8), ch = task % (C::DV / 8);
-        if (task < C::V_TASKS) {
-            const int col = slot_of(quad * 4); // 4 keys stay adjacent, quads are permuted
+        for (int i = 0; i < C::K_PT; ++i) st.k[i] = *reinterpret_cast<const u32x4_t *>(kt + koff[i]);
+        if constexpr (C::NKR > 0) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { // channel ch*8 + e gets the four keys as one 8-byte store
-                const int w = e >> 1, sh = (e & 1) * 16;
-                u32x2_t pk;
-                pk[0] = ((st.v[i][0][w] >> sh) & 0xffffu) | (((st.v[i][1][w] >> sh) & 0xffffu) << 16);
-                pk[1] = ((st.v[i][2][w] >> sh) & 0xffffu) | (((st.v[i][3][w] >> sh) & 0xffffu) << 16);
-                *reinterpret_cast<u32x2_t *>(sVt + (ch * 8 + e) * C::BNP + col) = pk;
+            for (int i = 0; i < C::KB_PT; ++i) st.kb[i] = *reinterpret_cast<const u32x4_t *>(kbt + kboff[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) st.v[i][j] = *reinterpret_cast<const u32x2_t *>(vt + voff[i][j]);
+    }
+
+    // Any tile: rows past the end and columns past d / r read a clamped address and become 0.
+    __device__ __forceinline__ void load_safe(FwdStage<C> &st, const FwdArgs &a, const uint16_t *kbase,
+                                              const uint16_t *kbbase, const uint16_t *vbase, int n0, int tid) const {
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            st.k[i] = load_chunk<C::VEC>(kbase, a.k.ss, n0 + task % C::BN, a.Lk, (task / C::BN) * 8, a.d);
+        }
+        if constexpr (C::NKR > 0) {
+#pragma unroll
+            for (int i = 0; i < C::KB_PT; ++i) {
+                const int task = tid + i * C::NTHREADS;
+                st.kb[i] = load_chunk<C::VEC>(kbbase, a.kb.ss, n0 + task % C::BN, a.Lk, (task / C::BN) * 8, a.r);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) {
+            const int task = (C::NTHREADS - 1 - tid) + i * C::NTHREADS;
+            const int quad = task % (C::BN / 4), hc = task / (C::BN / 4);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                st.v[i][j] = load_half<C::VEC>(vbase, a.v.ss, n0 + quad * 4 + j, a.Lk, hc * 4, a.d);
+        }
+    }
+
+    // Registers -> LDS.  Threads whose chunk lies in the zero padding of the channel dimension
+    // never store: those LDS columns are cleared once before the loop.
+    __device__ __forceinline__ void store(const FwdStage<C> &st, uint16_t *sK, uint16_t *sVt) const {
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i)
+            if (kok[i]) *reinterpret_cast<u32x4_t *>(sK + kdst[i]) = st.k[i];
+        if constexpr (C::NKR > 0) {
+#pragma unroll
+            for (int i = 0; i < C::KB_PT; ++i)
+                if (kbok[i]) *reinterpret_cast<u32x4_t *>(sK + kbdst[i]) = st.kb[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) {
+            if (vok[i]) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { // channel hc*4 + e gets its four keys as one 8-byte store
+                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                    u32x2_t pk;
+                    pk[0] = __builtin_amdgcn_perm(st.v[i][1][e >> 1], st.v[i][0][e >> 1], sel);
+                    pk[1] = __builtin_amdgcn_perm(st.v[i][3][e >> 1], st.v[i][2][e >> 1], sel);
+                    *reinterpret_cast<u32x2_t *>(sVt + vdst[i] + e * C::BNP) = pk;
+                }
             }
         }
     }
-}
+};
 
 // Additive mask value for (query, key); 0 outside the tensor (those scores are -inf anyway).
 template <class T>
@@ -124,7 +202,8 @@ __device__ __forceinline__ float mask_at(const MaskDesc &m, const uint8_t *base,
 }
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 3))) void fwd_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, C::WAVES_EU))) void fwd_kernel(
+    const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *sKbuf = reinterpret_cast<uint16_t *>(smem);
     uint16_t *sVbuf = sKbuf + 2 * C::SK_ELEMS;
@@ -139,7 +218,8 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
-    const int wq0 = m0 + wave * (32 * C::QBLK); // first query of this wave
+    const int wq0 = m0 + wave * 32; // first query of this wave
+    const int query = wq0 + c;
 
     const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
     const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
@@ -155,85 +235,89 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
     // ---- query operand, resident in registers for the whole key loop
-    u32x4_t qreg[C::QBLK][C::NK];
+    u32x4_t qhi[C::NKD], qlo[C::NKD], qbr[C::NKR > 0 ? C::NKR : 1];
 #pragma unroll
-    for (int qb = 0; qb < C::QBLK; ++qb) {
-        const int query = wq0 + qb * 32 + c;
+    for (int t = 0; t < C::NKD; ++t)
+        split_scaled<T>(load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d), a.scale, qhi[t], qlo[t]);
+    if constexpr (C::NKR > 0) {
 #pragma unroll
-        for (int t = 0; t < C::NK; ++t) {
-            if (t < C::NKD)
-                qreg[qb][t] = load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d);
-            else if constexpr (C::NKR > 0)
-                qreg[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * (t - C::NKD) + 8 * g, a.r);
-        }
+        for (int t = 0; t < C::NKR; ++t)
+            qbr[t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * t + 8 * g, a.r);
     }
 
-    f32x16_t acc_o[C::QBLK][C::NDV];
-    float m_run[C::QBLK], l_run[C::QBLK]; // running max (natural units), per-lane partial row sum
+    f32x16_t acc_o[C::NDV];
 #pragma unroll
-    for (int qb = 0; qb < C::QBLK; ++qb) {
-        m_run[qb] = -INFINITY;
-        l_run[qb] = 0.f;
+    for (int n = 0; n < C::NDV; ++n)
 #pragma unroll
-        for (int n = 0; n < C::NDV; ++n)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc_o[qb][n][v] = 0.f;
-    }
+        for (int v = 0; v < 16; ++v) acc_o[n][v] = 0.f;
+    float m_ref = -INFINITY; // reference of the exponentials (natural units), lags the true row max
+    float m2 = 0.f;          // m_ref * log2(e), 0 while the row has seen no finite score
+    float l_run = 0.f;       // per-lane partial row sum (the two lanes of a query are added at the end)
+    constexpr float kLagNat = 8.0f * kLn2; // let the row max run ahead of m_ref by up to 2^8
 
     // causal: tiles past the last query of this workgroup are never visible (:202)
     int k_end = a.Lk;
     if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM;
     const int ntiles_k = (k_end + C::BN - 1) / C::BN;
 
+    FwdLoader<C> ld;
+    ld.init(a, tid);
+    {   // clear both LDS buffers once: the zero padding of the channel dimension is never rewritten
+        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
+        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+    auto load_tile = [&](FwdStage<C> &stg, int n0) {
+        if (C::VEC && n0 + C::BN <= a.Lk)
+            ld.load_fast(stg, kbase + (int64_t)n0 * a.k.ss, C::NKR > 0 ? kbbase + (int64_t)n0 * a.kb.ss : nullptr,
+                         vbase + (int64_t)n0 * a.v.ss);
+        else
+            ld.load_safe(stg, a, kbase, kbbase, vbase, n0, tid);
+    };
     FwdStage<C> st;
-    fwd_load_tile<C>(st, a, kbase, kbbase, vbase, 0, tid);
-    fwd_store_tile<C>(st, sKbuf, sVbuf, tid);
+    load_tile(st, 0);
+    ld.store(st, sKbuf, sVbuf);
     __syncthreads();
 
     for (int it = 0; it < ntiles_k; ++it) {
         const int cur = it & 1;
         const int n0 = it * C::BN;
         const bool more = it + 1 < ntiles_k;
-        if (more) fwd_load_tile<C>(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
+        if (more) load_tile(st, n0 + C::BN);
 
         const uint16_t *sK = sKbuf + cur * C::SK_ELEMS;
         const uint16_t *sVt = sVbuf + cur * C::SV_ELEMS;
-        const int wq_last = wq0 + 32 * C::QBLK - 1;
-        const bool visible = !(a.causal && n0 > wq_last) && wq0 < a.Lq;
+        const bool visible = !(a.causal && n0 > wq0 + 31) && wq0 < a.Lq;
         if (visible) {
-            // ---- S^T = [K | K_b] [Q | Q_b]^T
-            f32x16_t s[C::KBLK][C::QBLK];
+            // ---- S^T = [K | K_b] [scale Q | Q_b]^T
+            f32x16_t s[C::KBLK];
 #pragma unroll
             for (int kb = 0; kb < C::KBLK; ++kb) {
-                u32x4_t ka[C::NK];
+                f32x16_t acc;
 #pragma unroll
-                for (int t = 0; t < C::NK; ++t)
-                    ka[t] = *reinterpret_cast<const u32x4_t *>(sK + (kb * 32 + c) * C::DKP + 16 * t + 8 * g);
+                for (int v = 0; v < 16; ++v) acc[v] = 0.f;
 #pragma unroll
-                for (int qb = 0; qb < C::QBLK; ++qb) {
-                    f32x16_t acc;
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-#pragma unroll
-                    for (int t = 0; t < C::NKD; ++t) acc = T::mfma(ka[t], qreg[qb][t], acc);
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[v] *= a.scale;
-#pragma unroll
-                    for (int t = C::NKD; t < C::NK; ++t) acc = T::mfma(ka[t], qreg[qb][t], acc);
-                    s[kb][qb] = acc;
+                for (int t = 0; t < C::NK; ++t) {
+                    const u32x4_t ka =
+                        *reinterpret_cast<const u32x4_t *>(sK + (kb * 32 + c) * C::DKP + 16 * t + 8 * g);
+                    if (t < C::NKD) {
+                        acc = T::mfma(ka, qhi[t], acc);
+                        acc = T::mfma(ka, qlo[t], acc);
+                    } else {
+                        acc = T::mfma(ka, qbr[t - C::NKD], acc);
+                    }
                 }
+                s[kb] = acc;
             }
             // ---- additive mask, then -inf for keys past the end and causal-hidden pairs
             if constexpr (C::MASK) {
 #pragma unroll
                 for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
-                    for (int qb = 0; qb < C::QBLK; ++qb)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
-                            s[kb][qb][v] += mask_at<T>(a.mask, mbase, wq0 + qb * 32 + c, key, a.Lq, a.Lk);
-                        }
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                        s[kb][v] += mask_at<T>(a.mask, mbase, query, key, a.Lq, a.Lk);
+                    }
             }
             const bool ragged = n0 + C::BN > a.Lk;
             const bool diag = a.causal && (n0 + C::BN - 1 > wq0);
@@ -241,100 +325,84 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
                 for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
-                    for (int qb = 0; qb < C::QBLK; ++qb)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
-                            const int query = wq0 + qb * 32 + c;
-                            if (key >= a.Lk || (a.causal && key > query)) s[kb][qb][v] = -INFINITY;
-                        }
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                        if (key >= a.Lk || (a.causal && key > query)) s[kb][v] = -INFINITY;
+                    }
             }
             // ---- online softmax, one query per lane (two lanes share a query)
+            float mx = s[0][0];
 #pragma unroll
-            for (int qb = 0; qb < C::QBLK; ++qb) {
-                float mx = m_run[qb];
+            for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
-                for (int kb = 0; kb < C::KBLK; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kb][qb][v]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float mref = (mx == -INFINITY) ? 0.f : mx; // whole row hidden so far
-                const float m2 = mref * kLog2e;
-                const float alpha = fast_exp2(m_run[qb] * kLog2e - m2);
-                float lsum = 0.f;
-#pragma unroll
-                for (int kb = 0; kb < C::KBLK; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const float p = fast_exp2(__builtin_fmaf(s[kb][qb][v], kLog2e, -m2));
-                        s[kb][qb][v] = p;
-                        lsum += p;
-                    }
-                l_run[qb] = l_run[qb] * alpha + lsum;
-                m_run[qb] = mx;
+                for (int v = (kb == 0 ? 1 : 0); v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const bool grow = mx > m_ref + kLagNat; // also true for the first finite score of a row
+            if (__any(grow)) {
+                const float m_new = grow ? mx : m_ref;
+                const float alpha = grow ? fast_exp2((m_ref - m_new) * kLog2e) : 1.f; // exp2(-inf) = 0
+                l_run *= alpha;
 #pragma unroll
                 for (int n = 0; n < C::NDV; ++n)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc_o[qb][n][v] *= alpha;
+                    for (int v = 0; v < 16; ++v) acc_o[n][v] *= alpha;
+                m_ref = m_new;
+                m2 = (m_ref == -INFINITY) ? 0.f : m_ref * kLog2e;
             }
-            // ---- O^T += V^T P^T
+            // ---- P^T = exp(S^T - m_ref), row sums, O^T += V^T P^T
 #pragma unroll
             for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    u32x4_t pb[C::QBLK];
+                    u32x4_t pb;
 #pragma unroll
-                    for (int qb = 0; qb < C::QBLK; ++qb)
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            pb[qb][e] = T::pack2(s[kb][qb][8 * t + 2 * e], s[kb][qb][8 * t + 2 * e + 1]);
+                    for (int e = 0; e < 4; ++e) {
+                        const float p0 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e], kLog2e, -m2));
+                        const float p1 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e + 1], kLog2e, -m2));
+                        pb[e] = T::pack2(p0, p1);
+                        l_run = T::dot2_ones(pb[e], l_run);
+                    }
 #pragma unroll
                     for (int n = 0; n < C::NDV; ++n) {
                         const u32x4_t va = *reinterpret_cast<const u32x4_t *>(
                             sVt + (32 * n + c) * C::BNP + kb * 32 + 16 * t + 8 * g);
-#pragma unroll
-                        for (int qb = 0; qb < C::QBLK; ++qb) acc_o[qb][n] = T::mfma(va, pb[qb], acc_o[qb][n]);
+                        acc_o[n] = T::mfma(va, pb, acc_o[n]);
                     }
                 }
         }
-        if (more) fwd_store_tile<C>(st, sKbuf + (cur ^ 1) * C::SK_ELEMS, sVbuf + (cur ^ 1) * C::SV_ELEMS, tid);
+        if (more) ld.store(st, sKbuf + (cur ^ 1) * C::SK_ELEMS, sVbuf + (cur ^ 1) * C::SV_ELEMS);
         __syncthreads();
     }
 
-    // ---- epilogue: o = acc / l, lse = m + ln(l)
+    // ---- epilogue: o = acc / l, lse = m_ref + ln(l)
     uint16_t *obase = const_cast<uint16_t *>(a.o.ptr) + b * a.o.sb + h * a.o.sh;
+    const float l = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = 1.f / l;
+    if (query < a.Lq) {
+        if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref + __builtin_amdgcn_logf(l) * kLn2;
+        uint16_t *orow = obase + (int64_t)query * a.o.ss;
 #pragma unroll
-    for (int qb = 0; qb < C::QBLK; ++qb) {
-        const int query = wq0 + qb * 32 + c;
-        const float l = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
-        const float inv = 1.f / l;
-        if (query < a.Lq) {
-            if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_run[qb] + __builtin_amdgcn_logf(l) * kLn2;
-            uint16_t *orow = obase + (int64_t)query * a.o.ss;
+        for (int n = 0; n < C::NDV; ++n)
 #pragma unroll
-            for (int n = 0; n < C::NDV; ++n)
+            for (int bq = 0; bq < 4; ++bq) {
+                const int ch = 32 * n + 8 * bq + 4 * g;
+                if (C::VEC && ch + 4 <= a.d) {
+                    u32x2_t pk;
+                    pk[0] = T::pack2(acc_o[n][4 * bq] * inv, acc_o[n][4 * bq + 1] * inv);
+                    pk[1] = T::pack2(acc_o[n][4 * bq + 2] * inv, acc_o[n][4 * bq + 3] * inv);
+                    *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
+                } else {
 #pragma unroll
-                for (int bq = 0; bq < 4; ++bq) {
-                    const int ch = 32 * n + 8 * bq + 4 * g;
-                    if (C::VEC && ch + 4 <= a.d) {
-                        u32x2_t pk;
-                        pk[0] = T::pack2(acc_o[qb][n][4 * bq] * inv, acc_o[qb][n][4 * bq + 1] * inv);
-                        pk[1] = T::pack2(acc_o[qb][n][4 * bq + 2] * inv, acc_o[qb][n][4 * bq + 3] * inv);
-                        *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (ch + e < a.d) orow[ch + e] = T::from_float(acc_o[qb][n][4 * bq + e] * inv);
-                    }
+                    for (int e = 0; e < 4; ++e)
+                        if (ch + e < a.d) orow[ch + e] = T::from_float(acc_o[n][4 * bq + e] * inv);
                 }
-        }
+            }
     }
 }
 
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
 static hipError_t launch_fwd_vec(const FwdArgs &a0, hipStream_t stream) {
-    constexpr int QBLK = 1;
-    typedef FwdCfg<T, NKD, NKR, NDV, QBLK, VEC, MASK> C;
+    typedef FwdCfg<T, NKD, NKR, NDV, VEC, MASK> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_kernel<T, C>;
