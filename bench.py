@@ -8,7 +8,7 @@ line:
 
   value        whole-step throughput in TFLOP/s, algorithmic FLOPs 2 B H L^2 (7d + 4r)
   ms_per_step  forward + backward wall time per step
-  roofline     the dominant kernel (backward main) timed alone with events on its stream,
+  roofline     the dominant kernel (backward dk/dv) timed alone with events on its stream,
                against the dense bf16 MFMA peak
   cpu_baseline the eager oracle (restated reference eager attention) on the host cores, on a
                bounded sample of the same workload
@@ -68,17 +68,15 @@ def _phase_timers(w, dev):
         p.dq_bias, p.dk_bias = _tensor(full[0]), _tensor(full[1])
         keep += full
     delta = torch.empty_like(lse)
-    nbytes = lib.fb_bwd_workspace_bytes(p)
-    ws = torch.empty(nbytes // 4, device=dev, dtype=torch.float32)
-    p.delta, p.workspace, p.workspace_bytes = delta.data_ptr(), ws.data_ptr(), nbytes
-    keep += [o, lse, grads, delta, ws]
+    p.delta = delta.data_ptr()
+    keep += [o, lse, grads, delta]
 
     def call(fn):
         def run():
             _lib.check_status(fn(p, _stream()))
         return run
     return {name: call(getattr(lib, name)) for name in
-            ("fb_fwd", "fb_bwd_preprocess", "fb_bwd_main", "fb_bwd_finalize")}, keep
+            ("fb_fwd", "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq")}, keep
 
 
 def _cpu_baseline(w, flops_per_slice):
@@ -128,9 +126,11 @@ def headline(args):
     f_fwd, f_bwd = workloads.flops(hl["B"], hl["H"], hl["L"], hl["L"], hl["d"], hl["r"])
     phases, keep = _phase_timers({n: (t.detach() if isinstance(t, torch.Tensor) else t) for n, t in w.items()}, dev)
     ms = {name: _time_events(fn, args.steps, max(1, args.warmup)) for name, fn in phases.items()}
-    # the backward main kernel: everything of the backward except delta (2 B H L d) and the casts
-    f_main = f_bwd
-    tflops_main = f_main / (ms["fb_bwd_main"] * 1e-3) / 1e12
+    # dominant kernel: dk/dv/dk_bias.  Its algorithmic share of the backward: S recompute
+    # (d + r), dP (d), dV (d), dK|dK_b (d + r) of the 2 B H L^2 (5d + 3r); the dq kernel carries
+    # the dQ|dQ_b product (d + r) and, beyond the algorithmic count, a second S / dP recompute.
+    f_dkv = 2.0 * hl["B"] * hl["H"] * hl["L"] * hl["L"] * (4 * hl["d"] + 2 * hl["r"])
+    tflops_main = f_dkv / (ms["fb_bwd_dkv"] * 1e-3) / 1e12
     value = (f_fwd + f_bwd) / (ms_step * 1e-3) / 1e12
     ref_fwd, ref_fb = workloads.reference_formula_flops(hl["B"], hl["H"], hl["L"], hl["d"])
     out = {
@@ -151,10 +151,10 @@ def headline(args):
         "pct_of_bf16_mfma_peak": round(100 * value / PEAK_BF16_TFLOPS, 2),
         "fwd_ms": round(ms["fb_fwd"], 4),
         "fwd_tflops": round(f_fwd / (ms["fb_fwd"] * 1e-3) / 1e12, 2),
-        "bwd_ms": round(ms["fb_bwd_preprocess"] + ms["fb_bwd_main"] + ms["fb_bwd_finalize"], 4),
+        "bwd_ms": round(ms["fb_bwd_preprocess"] + ms["fb_bwd_dkv"] + ms["fb_bwd_dq"], 4),
         "kernel_ms": {k: round(v, 4) for k, v in ms.items()},
         "reference_formula_tflops": round(ref_fb / (ms_step * 1e-3) / 1e12, 2),
-        "roofline": {"kernel": "bwd_kernel (fb_bwd_main)", "bound": "mfma", "achieved": round(tflops_main, 2),
+        "roofline": {"kernel": "bwd_dkv_kernel (fb_bwd_dkv)", "bound": "mfma", "achieved": round(tflops_main, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_main / PEAK_BF16_TFLOPS, 4),
                      "traffic": None},
     }
@@ -181,7 +181,7 @@ def report(args):
         f_fwd, f_bwd = workloads.flops(B, H, Lq, w["k"].shape[1], d, r, w["causal"])
         phases, keep = _phase_timers(w, dev)
         ms = {n: _time_events(fn, args.steps, args.warmup) for n, fn in phases.items()}
-        bwd = ms["fb_bwd_preprocess"] + ms["fb_bwd_main"] + ms["fb_bwd_finalize"]
+        bwd = ms["fb_bwd_preprocess"] + ms["fb_bwd_dkv"] + ms["fb_bwd_dq"]
         rows.append((name, ms["fb_fwd"], f_fwd / ms["fb_fwd"] / 1e9, ms["fb_fwd"] + bwd,
                      (f_fwd + f_bwd) / (ms["fb_fwd"] + bwd) / 1e9))
         del keep, w

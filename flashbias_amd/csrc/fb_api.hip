@@ -11,7 +11,8 @@
 namespace fb {
 #define FB_DECL(sfx)                                                          \
     hipError_t launch_fwd_##sfx(const FwdArgs &a, hipStream_t stream);        \
-    hipError_t launch_bwd_main_##sfx(const BwdArgs &a, hipStream_t stream);
+    hipError_t launch_bwd_dkv_##sfx(const BwdArgs &a, hipStream_t stream);    \
+    hipError_t launch_bwd_dq_##sfx(const BwdArgs &a, hipStream_t stream);
 FB_DECL(bf16_1) FB_DECL(bf16_2) FB_DECL(bf16_4) FB_DECL(bf16_8)
 FB_DECL(f16_1) FB_DECL(f16_2) FB_DECL(f16_4) FB_DECL(f16_8)
 #undef FB_DECL
@@ -25,12 +26,21 @@ hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream) {
     }
 }
 
-hipError_t launch_bwd_main(const BwdArgs &a, bool bf16, hipStream_t stream) {
+hipError_t launch_bwd_dkv(const BwdArgs &a, bool bf16, hipStream_t stream) {
     switch (nkd_of(a.d)) {
-    case 1: return bf16 ? launch_bwd_main_bf16_1(a, stream) : launch_bwd_main_f16_1(a, stream);
-    case 2: return bf16 ? launch_bwd_main_bf16_2(a, stream) : launch_bwd_main_f16_2(a, stream);
-    case 4: return bf16 ? launch_bwd_main_bf16_4(a, stream) : launch_bwd_main_f16_4(a, stream);
-    default: return bf16 ? launch_bwd_main_bf16_8(a, stream) : launch_bwd_main_f16_8(a, stream);
+    case 1: return bf16 ? launch_bwd_dkv_bf16_1(a, stream) : launch_bwd_dkv_f16_1(a, stream);
+    case 2: return bf16 ? launch_bwd_dkv_bf16_2(a, stream) : launch_bwd_dkv_f16_2(a, stream);
+    case 4: return bf16 ? launch_bwd_dkv_bf16_4(a, stream) : launch_bwd_dkv_f16_4(a, stream);
+    default: return bf16 ? launch_bwd_dkv_bf16_8(a, stream) : launch_bwd_dkv_f16_8(a, stream);
+    }
+}
+
+hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream) {
+    switch (nkd_of(a.d)) {
+    case 1: return bf16 ? launch_bwd_dq_bf16_1(a, stream) : launch_bwd_dq_f16_1(a, stream);
+    case 2: return bf16 ? launch_bwd_dq_bf16_2(a, stream) : launch_bwd_dq_f16_2(a, stream);
+    case 4: return bf16 ? launch_bwd_dq_bf16_4(a, stream) : launch_bwd_dq_f16_4(a, stream);
+    default: return bf16 ? launch_bwd_dq_bf16_8(a, stream) : launch_bwd_dq_f16_8(a, stream);
     }
 }
 } // namespace fb
@@ -87,8 +97,6 @@ int check_out(const fb_tensor &t, int channels, int B, int H, int L, const char 
     return FB_OK;
 }
 
-uint64_t lq_pad_of(const fb_params *p) { return (static_cast<uint64_t>(p->Lq) + 31) / 32 * 32; }
-
 fb::FwdArgs fwd_args(const fb_params *p) {
     fb::FwdArgs a;
     std::memset(&a, 0, sizeof(a));
@@ -128,10 +136,6 @@ fb::BwdArgs bwd_args(const fb_params *p) {
     a.mask = dev_mask(p);
     a.lse = p->lse;
     a.delta = p->delta;
-    a.dq_acc = static_cast<float *>(p->workspace);
-    a.lq_pad = static_cast<int64_t>(lq_pad_of(p));
-    a.dq_rows = p->d + p->r;
-    a.r_row0 = p->d;
     a.B = p->B; a.H = p->H; a.Lq = p->Lq; a.Lk = p->Lk; a.d = p->d; a.r = p->r;
     a.causal = p->causal ? 1 : 0;
     a.scale = p->scale;
@@ -151,11 +155,6 @@ extern "C" {
 int fb_version(void) { return FB_VERSION; }
 
 const char *fb_last_error(void) { return g_err; }
-
-uint64_t fb_bwd_workspace_bytes(const fb_params *p) {
-    if (!p || p->B <= 0 || p->H <= 0 || p->Lq <= 0 || p->d <= 0 || p->r < 0) return 0;
-    return static_cast<uint64_t>(p->B) * p->H * (p->d + p->r) * lq_pad_of(p) * sizeof(float);
-}
 
 int fb_check(const fb_params *p, int pass) {
     g_err[0] = 0;
@@ -195,10 +194,6 @@ int fb_check(const fb_params *p, int pass) {
         if ((rc = check_out(p->dk_bias, p->r, p->B, p->H, p->Lk, "dk_bias"))) return rc;
     }
     if (!p->delta) return fail(FB_ERR_NULL, "%s: null pointer", "delta");
-    if (!p->workspace || p->workspace_bytes < fb_bwd_workspace_bytes(p))
-        return fail(FB_ERR_WORKSPACE, "workspace missing or smaller than fb_bwd_workspace_bytes()");
-    if (reinterpret_cast<uintptr_t>(p->workspace) % 16 != 0)
-        return fail(FB_ERR_WORKSPACE, "workspace must be 16-byte aligned");
     return FB_OK;
 }
 
@@ -215,25 +210,25 @@ int fb_bwd_preprocess(const fb_params *p, void *stream) {
                     "fb_bwd_preprocess");
 }
 
-int fb_bwd_main(const fb_params *p, void *stream) {
+int fb_bwd_dkv(const fb_params *p, void *stream) {
     const int rc = fb_check(p, 1);
     if (rc) return rc;
-    return launched(fb::launch_bwd_main(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
-                    "fb_bwd_main");
+    return launched(fb::launch_bwd_dkv(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                    "fb_bwd_dkv");
 }
 
-int fb_bwd_finalize(const fb_params *p, void *stream) {
+int fb_bwd_dq(const fb_params *p, void *stream) {
     const int rc = fb_check(p, 1);
     if (rc) return rc;
-    return launched(fb::launch_bwd_finalize(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
-                    "fb_bwd_finalize");
+    return launched(fb::launch_bwd_dq(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                    "fb_bwd_dq");
 }
 
 int fb_bwd(const fb_params *p, void *stream) {
     int rc = fb_bwd_preprocess(p, stream);
     if (rc) return rc;
-    if ((rc = fb_bwd_main(p, stream))) return rc;
-    return fb_bwd_finalize(p, stream);
+    if ((rc = fb_bwd_dkv(p, stream))) return rc;
+    return fb_bwd_dq(p, stream);
 }
 
 } // extern "C"

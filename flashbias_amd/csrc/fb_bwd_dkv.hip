@@ -1,0 +1,416 @@
+// Backward FlashBias attention for gfx950, part 1 of 2: dk, dv and dk_bias.
+// Together with fb_bwd_dq.hip this replaces _bwd_kernel of the reference
+// (flash_bias/flash_bias_triton.py:450-1097); this kernel covers the key-block loop of
+// _bwd_kernel_one_col_block (:575-869) except its dq / dq_bias updates.
+//
+// Key-stationary: one workgroup (4 waves) owns 64 * KBW consecutive keys of one
+// (batch, head), wave w owns KBW blocks of 32 of them, whose K, K_b and V stay in registers.
+// Queries are streamed in steps of 64 (two 32-blocks) through double-buffered LDS, the next
+// step prefetched into registers.  With lane = key, register = query (C layout of S with A = query rows from
+// LDS, B = key registers):
+//
+//   S   = [Q | Q_b] [K | K_b]^T, the q k^T part times scale  (:638-641)
+//   P   = exp(S - lse)                                         (:670)
+//   dP  = dO V^T - delta      accumulator starts at -delta, read from LDS into place (:705-714)
+//   dS  = P * dP
+//   dV^T          += dO^T P              A = dO^T tile (LDS),      B = P registers   (:697)
+//   [dK | dK_b]^T += [Q | Q_b]^T dS      A = [Q | Q_b]^T tile (LDS), B = dS registers (:717-719)
+//
+// P and dS feed their MFMAs straight from the accumulator layout (no LDS round trip); every
+// A operand read from LDS is used for all KBW key blocks of the wave.  The accumulators are
+// summed in a fixed order: dk, dv, dk_bias are bit-reproducible.
+#include "fb_kernels.h"
+
+namespace fb {
+
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_>
+struct DkvCfg {
+    static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
+    static constexpr bool VEC = VEC_, MASK = MASK_;
+    static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
+    static constexpr int NK = NKD + NKR;
+    static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dK | dK_b]^T
+    static constexpr int KBW = (NK <= 4 && NDV <= 1) ? 2 : 1; // key blocks per wave
+    static constexpr int BN = 32 * KBW * NWAVES;              // keys per workgroup
+    static constexpr int QBLK = 2, BMQ = 32 * QBLK;           // queries per step
+    static constexpr int DKP = 16 * NK + 8;  // sQ row (elements)
+    static constexpr int DOP = 16 * NKD + 8; // sdO row
+    static constexpr int QTP = BMQ + 8;      // sQt / sdOt row (queries, slot-permuted)
+    static constexpr int SQ = BMQ * DKP, SDO = BMQ * DOP, SQT = 32 * MB * QTP, SDOT = 32 * NDV * QTP;
+    static constexpr int STAGE_ELEMS = SQ + SDO + SQT + SDOT + 4 * BMQ; // + lse2, -delta as fp32
+    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2; // two stages
+    // loader tasks: (4 queries x 8 channels) blocks of Q, Q_b and dout
+    static constexpr int CQ = 2 * NKD, CR = 2 * NKR, CO = 2 * NKD;
+    static constexpr int QUADS = BMQ / 4;
+    static constexpr int TASKS = QUADS * (CQ + CR + CO);
+    static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
+    static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 2 : 1;
+};
+
+template <class C>
+struct DkvStage {
+    u32x4_t x[C::PT][4];
+    float lse2, negd;
+};
+
+// task -> (kind, quad, chunk): kind 0 = Q, 1 = Q_b, 2 = dout
+template <class C>
+__device__ __forceinline__ void dkv_task(int task, int &kind, int &quad, int &ch) {
+    quad = task % C::QUADS;
+    const int cc = task / C::QUADS;
+    if (cc < C::CQ) {
+        kind = 0;
+        ch = cc;
+    } else if (cc < C::CQ + C::CR) {
+        kind = 1;
+        ch = cc - C::CQ;
+    } else {
+        kind = 2;
+        ch = cc - C::CQ - C::CR;
+    }
+}
+
+template <class C>
+__device__ __forceinline__ void dkv_load_step(DkvStage<C> &st, const BwdArgs &a, const uint16_t *qbase,
+                                              const uint16_t *qbbase, const uint16_t *dobase, const float *lse,
+                                              const float *delta, int m0, int tid) {
+#pragma unroll
+    for (int i = 0; i < C::PT; ++i) {
+        const int task = tid + i * C::NTHREADS;
+        int kind, quad, ch;
+        dkv_task<C>(task, kind, quad, ch);
+        // one load per task: pick the tensor by lane (all three share the chunk geometry)
+        const uint16_t *base = kind == 0 ? qbase : kind == 1 ? qbbase : dobase;
+        const int64_t ld = kind == 0 ? a.q.ss : kind == 1 ? a.qb.ss : a.dout.ss;
+        const int ncols = kind == 1 ? a.r : a.d;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            st.x[i][j] = u32x4_t{0u, 0u, 0u, 0u};
+            if (C::TASKS % C::NTHREADS == 0 || task < C::TASKS)
+                st.x[i][j] = load_chunk<C::VEC>(base, ld, m0 + quad * 4 + j, a.Lq, ch * 8, ncols);
+        }
+    }
+    st.lse2 = INFINITY; // rows past the end: P = exp2(-inf) = 0
+    st.negd = 0.f;
+    if (tid < C::BMQ && m0 + tid < a.Lq) {
+        st.lse2 = lse[m0 + tid] * kLog2e;
+        st.negd = -delta[m0 + tid];
+    }
+}
+
+template <class C>
+__device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *stage, int tid) {
+    uint16_t *sQ = stage, *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
+    float *sStat = reinterpret_cast<float *>(sdOt + C::SDOT);
+#pragma unroll
+    for (int i = 0; i < C::PT; ++i) {
+        const int task = tid + i * C::NTHREADS;
+        int kind, quad, ch;
+        dkv_task<C>(task, kind, quad, ch);
+        if (C::TASKS % C::NTHREADS == 0 || task < C::TASKS) {
+            // row-major copy (A operand of S and dP) ...
+            uint16_t *rm = kind == 2 ? sdO : sQ;
+            const int ld = kind == 2 ? C::DOP : C::DKP;
+            const int col0 = (kind == 1 ? 16 * C::NKD : 0) + ch * 8;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<u32x4_t *>(rm + (quad * 4 + j) * ld + col0) = st.x[i][j];
+            // ... and transposed copy (A operand of dV^T and [dK|dK_b]^T), queries slot-permuted
+            uint16_t *tr = kind == 2 ? sdOt : sQt;
+            const int qcol = slot_of(quad * 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                u32x2_t pk;
+                pk[0] = __builtin_amdgcn_perm(st.x[i][1][e >> 1], st.x[i][0][e >> 1], sel);
+                pk[1] = __builtin_amdgcn_perm(st.x[i][3][e >> 1], st.x[i][2][e >> 1], sel);
+                *reinterpret_cast<u32x2_t *>(tr + (col0 + e) * C::QTP + qcol) = pk;
+            }
+        }
+    }
+    if (tid < C::BMQ) {
+        sStat[tid] = st.lse2;
+        sStat[C::BMQ + tid] = st.negd;
+    }
+}
+
+template <class T>
+__device__ __forceinline__ float dkv_mask_at(const MaskDesc &m, const uint8_t *base, int query, int key, int Lq,
+                                             int Lk) {
+    if (key >= Lk || query >= Lq) return 0.f;
+    const int64_t off = (m.type == 2 ? (int64_t)query * m.sm : 0) + key;
+    if (m.is_f32) return reinterpret_cast<const float *>(base)[off];
+    return T::to_float(reinterpret_cast<const uint16_t *>(base)[off]);
+}
+
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU))) void
+bwd_dkv_kernel(const BwdArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 31, g = lane >> 5;
+
+    const int total = a.ntiles_n * a.B * a.H;
+    const int work = xcd_remap(blockIdx.x, total);
+    const int bh = work / a.ntiles_n;
+    const int tile_n = work % a.ntiles_n; // causal: low key tiles see the most queries, they go first
+    const int b = bh / a.H, h = bh % a.H;
+    const int n0 = tile_n * C::BN;
+    const int wk0 = n0 + wave * (32 * C::KBW); // first key of this wave
+
+    const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
+    const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
+    const uint16_t *vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
+    const uint16_t *dobase = a.dout.ptr + b * a.dout.sb + h * a.dout.sh;
+    const uint16_t *qbbase = nullptr, *kbbase = nullptr;
+    if constexpr (C::NKR > 0) {
+        qbbase = a.qb.ptr + b * a.qb.sb + h * a.qb.sh;
+        kbbase = a.kb.ptr + b * a.kb.sb + h * a.kb.sh;
+    }
+    const float *lse = a.lse + (int64_t)bh * a.Lq;
+    const float *delta = a.delta + (int64_t)bh * a.Lq;
+    const uint8_t *mbase = nullptr;
+    if constexpr (C::MASK)
+        mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
+                (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
+
+    // ---- key-side operands, resident in registers
+    u32x4_t kreg[C::KBW][C::NK];  // B operand of S: this lane's key, channels 16t + 8g ..
+    u32x4_t vreg[C::KBW][C::NKD]; // B operand of dP
+    f32x16_t acc_dv[C::KBW][C::NDV], acc_dk[C::KBW][C::MB];
+#pragma unroll
+    for (int kb = 0; kb < C::KBW; ++kb) {
+        const int key = wk0 + kb * 32 + c;
+#pragma unroll
+        for (int t = 0; t < C::NK; ++t) {
+            if (t < C::NKD)
+                kreg[kb][t] = load_chunk<C::VEC>(kbase, a.k.ss, key, a.Lk, 16 * t + 8 * g, a.d);
+            else if constexpr (C::NKR > 0)
+                kreg[kb][t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, 16 * (t - C::NKD) + 8 * g, a.r);
+        }
+#pragma unroll
+        for (int t = 0; t < C::NKD; ++t)
+            vreg[kb][t] = load_chunk<C::VEC>(vbase, a.v.ss, key, a.Lk, 16 * t + 8 * g, a.d);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+#pragma unroll
+            for (int n = 0; n < C::NDV; ++n) acc_dv[kb][n][v] = 0.f;
+#pragma unroll
+            for (int n = 0; n < C::MB; ++n) acc_dk[kb][n][v] = 0.f;
+        }
+    }
+
+    // causal: the first query step that can see this key tile (:498)
+    const int step0 = a.causal ? n0 / C::BMQ : 0;
+    const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
+
+    DkvStage<C> st;
+    if (step0 < nsteps) {
+        dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, step0 * C::BMQ, tid);
+        dkv_store_step<C>(st, stage0, tid);
+    }
+    __syncthreads();
+
+    for (int step = step0; step < nsteps; ++step) {
+        const int m0 = step * C::BMQ;
+        const int cur = (step - step0) & 1;
+        const bool more = step + 1 < nsteps;
+        if (more) dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, m0 + C::BMQ, tid);
+        const uint16_t *sQ = stage0 + cur * C::STAGE_ELEMS;
+        const uint16_t *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
+        const float *sStat = reinterpret_cast<const float *>(sdOt + C::SDOT);
+
+        const bool visible = !(a.causal && wk0 > m0 + C::BMQ - 1) && wk0 < a.Lk;
+        if (visible) {
+#pragma unroll
+            for (int qb = 0; qb < C::QBLK; ++qb) {
+                u32x4_t qa[C::NK], da[C::NKD];
+#pragma unroll
+                for (int t = 0; t < C::NK; ++t)
+                    qa[t] = *reinterpret_cast<const u32x4_t *>(sQ + (qb * 32 + c) * C::DKP + 16 * t + 8 * g);
+#pragma unroll
+                for (int t = 0; t < C::NKD; ++t)
+                    da[t] = *reinterpret_cast<const u32x4_t *>(sdO + (qb * 32 + c) * C::DOP + 16 * t + 8 * g);
+                u32x4_t pp[C::KBW][2], pds[C::KBW][2]; // P and dS, packed, per 16-query step
+#pragma unroll
+                for (int kb = 0; kb < C::KBW; ++kb) {
+                    const int key = wk0 + kb * 32 + c;
+                    f32x16_t s, dp;
+                    float lse2[16];
+                    // per-register query statistics: query = qb*32 + 8*(v/4) + 4g + v%4
+#pragma unroll
+                    for (int bq = 0; bq < 4; ++bq) {
+                        const f32x4_t l4 = *reinterpret_cast<const f32x4_t *>(sStat + qb * 32 + 8 * bq + 4 * g);
+                        const f32x4_t d4 =
+                            *reinterpret_cast<const f32x4_t *>(sStat + C::BMQ + qb * 32 + 8 * bq + 4 * g);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            lse2[4 * bq + e] = l4[e];
+                            dp[4 * bq + e] = d4[e];
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+                    for (int t = 0; t < C::NKD; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
+#pragma unroll
+                    for (int t = 0; t < C::NKD; ++t) dp = T::mfma(da[t], vreg[kb][t], dp);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] *= a.scale;
+#pragma unroll
+                    for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
+                    if constexpr (C::MASK) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            s[v] += dkv_mask_at<T>(a.mask, mbase, m0 + qb * 32 + 8 * (v >> 2) + 4 * g + (v & 3), key,
+                                                   a.Lq, a.Lk);
+                    }
+                    const bool edge = (wk0 + kb * 32 + 32 > a.Lk) || (a.causal && wk0 + kb * 32 + 31 > m0 + qb * 32);
+                    if (edge) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int query = m0 + qb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            if (key >= a.Lk || (a.causal && key > query)) s[v] = -INFINITY;
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[v]));
+                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[v + 1]));
+                        pp[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0, p1);
+                        pds[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
+                    }
+                }
+                // dV^T += dout^T P ; [dK|dK_b]^T += [Q|Q_b]^T dS  (contraction over this block's queries)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+#pragma unroll
+                    for (int n = 0; n < C::NDV; ++n) {
+                        const u32x4_t dot = *reinterpret_cast<const u32x4_t *>(sdOt + (32 * n + c) * C::QTP + qb * 32 +
+                                                                              16 * t + 8 * g);
+#pragma unroll
+                        for (int kb = 0; kb < C::KBW; ++kb) acc_dv[kb][n] = T::mfma(dot, pp[kb][t], acc_dv[kb][n]);
+                    }
+#pragma unroll
+                    for (int n = 0; n < C::MB; ++n) {
+                        const u32x4_t qt = *reinterpret_cast<const u32x4_t *>(sQt + (32 * n + c) * C::QTP + qb * 32 +
+                                                                             16 * t + 8 * g);
+#pragma unroll
+                        for (int kb = 0; kb < C::KBW; ++kb) acc_dk[kb][n] = T::mfma(qt, pds[kb][t], acc_dk[kb][n]);
+                    }
+                }
+            }
+        }
+        if (more) dkv_store_step<C>(st, stage0 + (cur ^ 1) * C::STAGE_ELEMS, tid);
+        __syncthreads();
+    }
+
+    // ---- epilogue: dv, dk (times scale), dk_bias for this lane's keys
+#pragma unroll
+    for (int kb = 0; kb < C::KBW; ++kb) {
+        const int key = wk0 + kb * 32 + c;
+        if (key < a.Lk) {
+            uint16_t *dvrow = const_cast<uint16_t *>(a.dv.ptr) + b * a.dv.sb + h * a.dv.sh + (int64_t)key * a.dv.ss;
+            uint16_t *dkrow = const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + (int64_t)key * a.dk.ss;
+            uint16_t *dkbrow = nullptr;
+            if constexpr (C::NKR > 0)
+                dkbrow = const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + (int64_t)key * a.dkb.ss;
+#pragma unroll
+            for (int n = 0; n < C::NDV; ++n)
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    const int ch = 32 * n + 8 * bq + 4 * g;
+                    if (C::VEC && a.dv.vec_ok && ch + 4 <= a.d) {
+                        u32x2_t pk;
+                        pk[0] = T::pack2(acc_dv[kb][n][4 * bq], acc_dv[kb][n][4 * bq + 1]);
+                        pk[1] = T::pack2(acc_dv[kb][n][4 * bq + 2], acc_dv[kb][n][4 * bq + 3]);
+                        *reinterpret_cast<u32x2_t *>(dvrow + ch) = pk;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (ch + e < a.d) dvrow[ch + e] = T::from_float(acc_dv[kb][n][4 * bq + e]);
+                    }
+                }
+#pragma unroll
+            for (int n = 0; n < C::MB; ++n)
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    const int ch = 32 * n + 8 * bq + 4 * g;
+                    if (ch < 16 * C::NKD) {
+                        if (C::VEC && a.dk.vec_ok && ch + 4 <= a.d) {
+                            u32x2_t pk;
+                            pk[0] = T::pack2(acc_dk[kb][n][4 * bq] * a.scale, acc_dk[kb][n][4 * bq + 1] * a.scale);
+                            pk[1] = T::pack2(acc_dk[kb][n][4 * bq + 2] * a.scale, acc_dk[kb][n][4 * bq + 3] * a.scale);
+                            *reinterpret_cast<u32x2_t *>(dkrow + ch) = pk;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (ch + e < a.d) dkrow[ch + e] = T::from_float(acc_dk[kb][n][4 * bq + e] * a.scale);
+                        }
+                    } else if constexpr (C::NKR > 0) {
+                        const int cr = ch - 16 * C::NKD;
+                        if (C::VEC && a.dkb.vec_ok && cr + 4 <= a.r) {
+                            u32x2_t pk;
+                            pk[0] = T::pack2(acc_dk[kb][n][4 * bq], acc_dk[kb][n][4 * bq + 1]);
+                            pk[1] = T::pack2(acc_dk[kb][n][4 * bq + 2], acc_dk[kb][n][4 * bq + 3]);
+                            *reinterpret_cast<u32x2_t *>(dkbrow + cr) = pk;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (cr + e < a.r) dkbrow[cr + e] = T::from_float(acc_dk[kb][n][4 * bq + e]);
+                        }
+                    }
+                }
+        }
+    }
+}
+
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+static hipError_t launch_dkv_vec(const BwdArgs &a0, hipStream_t stream) {
+    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK> C;
+    BwdArgs a = a0;
+    a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
+    auto kern = bwd_dkv_kernel<T, C>;
+    if (C::LDS_BYTES > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+    }
+    const int total = a.ntiles_n * a.B * a.H;
+    hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+    return hipGetLastError();
+}
+
+template <class T, int NKD, int NKR, int NDV>
+static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
+    const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+    if (a.mask.type)
+        return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, true>(a, stream)
+                   : launch_dkv_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, false>(a, stream)
+               : launch_dkv_vec<T, NKD, NKR, NDV, false, false>(a, stream);
+}
+
+template <class T, int NKD, int NDV>
+static hipError_t launch_dkv_r(const BwdArgs &a, hipStream_t stream) {
+    switch (nkr_of(a.r)) {
+    case 0: return launch_dkv_cfg<T, NKD, 0, NDV>(a, stream);
+    case 1: return launch_dkv_cfg<T, NKD, 1, NDV>(a, stream);
+    case 2: return launch_dkv_cfg<T, NKD, 2, NDV>(a, stream);
+    case 4: return launch_dkv_cfg<T, NKD, 4, NDV>(a, stream);
+    default: return launch_dkv_cfg<T, NKD, 8, NDV>(a, stream);
+    }
+}
+
+// Compiled once per (element type, head-dim bucket), see Makefile.
+#define FB_CAT2(a, b) a##b
+#define FB_CAT(a, b) FB_CAT2(a, b)
+hipError_t FB_CAT(launch_bwd_dkv_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
+    return launch_dkv_r<FB_T, FB_NKD, FB_NDV>(a, stream);
+}
+
+} // namespace fb

@@ -1,0 +1,369 @@
+// Backward FlashBias attention for gfx950, part 2 of 2: dq and dq_bias.
+// Together with fb_bwd_dkv.hip this replaces _bwd_kernel of the reference
+// (flash_bias/flash_bias_triton.py:450-1097); this kernel covers the dq / dq_bias updates of
+// :725-817 without their global read-modify-write or atomics.
+//
+// Query-stationary, like the forward: one workgroup (4 waves) owns 256 consecutive queries of
+// one (batch, head), each wave 64 of them (two 32-blocks); keys are streamed in tiles of 64
+// through double-buffered LDS.  With lane = query, register = key (transposed products):
+//
+//   S^T  = [K | K_b] [scale Q | Q_b]^T        A = key rows (LDS),        B = query registers
+//   dP^T = V dO^T - delta                     A = value rows (LDS),      B = dO registers,
+//                                             accumulator starts at -delta (a per-lane constant)
+//   P^T  = exp(S^T - lse)                     lse is a per-lane scalar
+//   dS^T = P^T * dP^T
+//   [dQ | dQ_b]^T += [K | K_b]^T dS^T         A = transposed key tile (LDS), B = dS^T registers
+//
+// so dS^T goes from the accumulator layout straight into the next MFMA and [dQ | dQ_b]^T stays
+// in registers for the whole key loop: each output element is written exactly once, in a fixed
+// summation order (bit-reproducible).  scale * q is split into hi + lo 16-bit parts as in the
+// forward; dq is multiplied by the scale in the epilogue, dq_bias is not (:728-732).
+#include "fb_kernels.h"
+
+namespace fb {
+
+template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_>
+struct DqCfg {
+    static constexpr int NKD = NKD_, NKR = NKR_;
+    static constexpr bool VEC = VEC_, MASK = MASK_;
+    static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
+    static constexpr int NK = NKD + NKR;
+    static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dQ | dQ_b]^T
+    static constexpr int QBLK = (NK <= 4) ? 2 : 1;
+    static constexpr int BM = NWAVES * QBLK * 32;
+    static constexpr int KBLK = 2, BN = 32 * KBLK;
+    static constexpr int DKP = 16 * NK + 8;  // sK row: [K | K_b] of one key
+    static constexpr int DVP = 16 * NKD + 8; // sV row: V of one key
+    static constexpr int BNP = BN + 8;       // sKt row: one channel, keys slot-permuted
+    static constexpr int SK = BN * DKP, SV = BN * DVP, SKT = 32 * MB * BNP;
+    static constexpr int STAGE = SK + SV + SKT;
+    static constexpr int LDS_BYTES = 2 * STAGE * 2;
+    // loader: (4 keys x 8 channels) blocks of K and K_b (written row-major and transposed),
+    // 8-channel chunks of V
+    static constexpr int CD = 2 * NKD, CR = 2 * NKR;
+    static constexpr int QUADS = BN / 4;
+    static constexpr int K_TASKS = QUADS * (CD + CR), V_TASKS = BN * CD;
+    static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
+    static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
+    static constexpr int WAVES_EU = (NK <= 4) ? 2 : 1;
+};
+
+template <class C>
+struct DqStage {
+    u32x4_t k[C::K_PT][4];
+    u32x4_t v[C::V_PT];
+};
+
+template <class C>
+struct DqLoader {
+    // K task: quad of 4 keys x one 8-channel chunk of K (chunk < CD) or K_b
+    __device__ static __forceinline__ void ktask(int task, int &quad, int &ch, bool &is_b) {
+        quad = task % C::QUADS;
+        const int cc = task / C::QUADS;
+        is_b = cc >= C::CD;
+        ch = is_b ? cc - C::CD : cc;
+    }
+
+    __device__ static __forceinline__ void load(DqStage<C> &st, const BwdArgs &a, const uint16_t *kbase,
+                                                const uint16_t *kbbase, const uint16_t *vbase, int n0, int tid) {
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            int quad, ch;
+            bool is_b;
+            ktask(task, quad, ch, is_b);
+            const uint16_t *base = is_b ? kbbase : kbase;
+            const int64_t ld = is_b ? a.kb.ss : a.k.ss;
+            const int ncols = is_b ? a.r : a.d;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                st.k[i][j] = u32x4_t{0u, 0u, 0u, 0u};
+                if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS)
+                    st.k[i][j] = load_chunk<C::VEC>(base, ld, n0 + quad * 4 + j, a.Lk, ch * 8, ncols);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            st.v[i] = u32x4_t{0u, 0u, 0u, 0u};
+            if (C::V_TASKS % C::NTHREADS == 0 || task < C::V_TASKS)
+                st.v[i] = load_chunk<C::VEC>(vbase, a.v.ss, n0 + task % C::BN, a.Lk, (task / C::BN) * 8, a.d);
+        }
+    }
+
+    __device__ static __forceinline__ void store(const DqStage<C> &st, uint16_t *stage, int tid) {
+        uint16_t *sK = stage, *sV = sK + C::SK, *sKt = sV + C::SV;
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            int quad, ch;
+            bool is_b;
+            ktask(task, quad, ch, is_b);
+            if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS) {
+                const int col0 = (is_b ? 16 * C::NKD : 0) + ch * 8;
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<u32x4_t *>(sK + (quad * 4 + j) * C::DKP + col0) = st.k[i][j];
+                const int kcol = slot_of(quad * 4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { // channel col0 + e gets its four keys as one 8-byte store
+                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
+                    u32x2_t pk;
+                    pk[0] = __builtin_amdgcn_perm(st.k[i][1][e >> 1], st.k[i][0][e >> 1], sel);
+                    pk[1] = __builtin_amdgcn_perm(st.k[i][3][e >> 1], st.k[i][2][e >> 1], sel);
+                    *reinterpret_cast<u32x2_t *>(sKt + (col0 + e) * C::BNP + kcol) = pk;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            if (C::V_TASKS % C::NTHREADS == 0 || task < C::V_TASKS)
+                *reinterpret_cast<u32x4_t *>(sV + (task % C::BN) * C::DVP + (task / C::BN) * 8) = st.v[i];
+        }
+    }
+};
+
+template <class T>
+__device__ __forceinline__ float dq_mask_at(const MaskDesc &m, const uint8_t *base, int query, int key, int Lq,
+                                            int Lk) {
+    if (key >= Lk || query >= Lq) return 0.f;
+    const int64_t off = (m.type == 2 ? (int64_t)query * m.sm : 0) + key;
+    if (m.is_f32) return reinterpret_cast<const float *>(base)[off];
+    return T::to_float(reinterpret_cast<const uint16_t *>(base)[off]);
+}
+
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU))) void
+bwd_dq_kernel(const BwdArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int c = lane & 31, g = lane >> 5;
+
+    const int total = a.ntiles_m * a.B * a.H;
+    const int work = xcd_remap(blockIdx.x, total);
+    const int bh = work / a.ntiles_m;
+    int tile_m = work % a.ntiles_m;
+    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
+    const int b = bh / a.H, h = bh % a.H;
+    const int m0 = tile_m * C::BM;
+    const int wq0 = m0 + wave * (32 * C::QBLK);
+
+    const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
+    const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
+    const uint16_t *vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
+    const uint16_t *dobase = a.dout.ptr + b * a.dout.sb + h * a.dout.sh;
+    const uint16_t *qbbase = nullptr, *kbbase = nullptr;
+    if constexpr (C::NKR > 0) {
+        qbbase = a.qb.ptr + b * a.qb.sb + h * a.qb.sh;
+        kbbase = a.kb.ptr + b * a.kb.sb + h * a.kb.sh;
+    }
+    const uint8_t *mbase = nullptr;
+    if constexpr (C::MASK)
+        mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
+                (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
+
+    // ---- query-side operands, resident in registers
+    u32x4_t qhi[C::QBLK][C::NKD], qlo[C::QBLK][C::NKD], qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
+    u32x4_t dor[C::QBLK][C::NKD];
+    f32x16_t negd[C::QBLK]; // -delta of this lane's query in every element: start of the dP^T accumulator
+    float lse2[C::QBLK];
+    f32x16_t acc[C::QBLK][C::MB];
+#pragma unroll
+    for (int qb = 0; qb < C::QBLK; ++qb) {
+        const int query = wq0 + qb * 32 + c;
+#pragma unroll
+        for (int t = 0; t < C::NKD; ++t) {
+            split_scaled<T>(load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d), a.scale, qhi[qb][t],
+                            qlo[qb][t]);
+            dor[qb][t] = load_chunk<C::VEC>(dobase, a.dout.ss, query, a.Lq, 16 * t + 8 * g, a.d);
+        }
+        if constexpr (C::NKR > 0) {
+#pragma unroll
+            for (int t = 0; t < C::NKR; ++t)
+                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * t + 8 * g, a.r);
+        }
+        const bool ok = query < a.Lq;
+        const int64_t sidx = (int64_t)bh * a.Lq + (ok ? query : a.Lq - 1);
+        lse2[qb] = ok ? a.lse[sidx] * kLog2e : INFINITY; // rows past the end: P = exp2(-inf) = 0
+        const float nd = ok ? -a.delta[sidx] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) negd[qb][v] = nd;
+#pragma unroll
+        for (int n = 0; n < C::MB; ++n)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[qb][n][v] = 0.f;
+    }
+
+    int k_end = a.Lk;
+    if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
+    const int ntiles_k = (k_end + C::BN - 1) / C::BN;
+
+    DqStage<C> st;
+    DqLoader<C>::load(st, a, kbase, kbbase, vbase, 0, tid);
+    DqLoader<C>::store(st, stage0, tid);
+    __syncthreads();
+
+    for (int it = 0; it < ntiles_k; ++it) {
+        const int cur = it & 1;
+        const int n0 = it * C::BN;
+        const bool more = it + 1 < ntiles_k;
+        if (more) DqLoader<C>::load(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
+
+        const uint16_t *sK = stage0 + cur * C::STAGE, *sV = sK + C::SK, *sKt = sV + C::SV;
+        const bool visible = !(a.causal && n0 > wq0 + 32 * C::QBLK - 1) && wq0 < a.Lq;
+        if (visible) {
+#pragma unroll
+            for (int kb = 0; kb < C::KBLK; ++kb) {
+                u32x4_t ka[C::NK], va[C::NKD];
+#pragma unroll
+                for (int t = 0; t < C::NK; ++t)
+                    ka[t] = *reinterpret_cast<const u32x4_t *>(sK + (kb * 32 + c) * C::DKP + 16 * t + 8 * g);
+#pragma unroll
+                for (int t = 0; t < C::NKD; ++t)
+                    va[t] = *reinterpret_cast<const u32x4_t *>(sV + (kb * 32 + c) * C::DVP + 16 * t + 8 * g);
+                u32x4_t dsp[C::QBLK][2]; // dS^T, packed, per 16-key step
+#pragma unroll
+                for (int qb = 0; qb < C::QBLK; ++qb) {
+                    f32x16_t s, dp = negd[qb];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+                    for (int t = 0; t < C::NK; ++t) {
+                        if (t < C::NKD) {
+                            s = T::mfma(ka[t], qhi[qb][t], s);
+                            s = T::mfma(ka[t], qlo[qb][t], s);
+                        } else {
+                            s = T::mfma(ka[t], qbr[qb][t - C::NKD], s);
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], dp);
+                    const int query = wq0 + qb * 32 + c;
+                    if constexpr (C::MASK) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            s[v] += dq_mask_at<T>(a.mask, mbase, query, n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3),
+                                                  a.Lq, a.Lk);
+                    }
+                    const bool edge = (n0 + kb * 32 + 32 > a.Lk) || (a.causal && n0 + kb * 32 + 31 > wq0 + qb * 32);
+                    if (edge) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            if (key >= a.Lk || (a.causal && key > query)) s[v] = -INFINITY;
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[qb]));
+                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[qb]));
+                        dsp[qb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
+                    }
+                }
+                // [dQ | dQ_b]^T += [K | K_b]^T dS^T over this block's 32 keys
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int n = 0; n < C::MB; ++n) {
+                        const u32x4_t kt = *reinterpret_cast<const u32x4_t *>(sKt + (32 * n + c) * C::BNP + kb * 32 +
+                                                                             16 * t + 8 * g);
+#pragma unroll
+                        for (int qb = 0; qb < C::QBLK; ++qb) acc[qb][n] = T::mfma(kt, dsp[qb][t], acc[qb][n]);
+                    }
+            }
+        }
+        if (more) DqLoader<C>::store(st, stage0 + (cur ^ 1) * C::STAGE, tid);
+        __syncthreads();
+    }
+
+    // ---- epilogue: dq = scale * acc rows [0, d), dq_bias = acc rows [16 NKD, 16 NKD + r)
+#pragma unroll
+    for (int qb = 0; qb < C::QBLK; ++qb) {
+        const int query = wq0 + qb * 32 + c;
+        if (query < a.Lq) {
+            uint16_t *dqrow = const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + (int64_t)query * a.dq.ss;
+            uint16_t *dqbrow = nullptr;
+            if constexpr (C::NKR > 0)
+                dqbrow = const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + (int64_t)query * a.dqb.ss;
+#pragma unroll
+            for (int n = 0; n < C::MB; ++n)
+#pragma unroll
+                for (int bq = 0; bq < 4; ++bq) {
+                    const int ch = 32 * n + 8 * bq + 4 * g; // 4 consecutive channels per lane
+                    if (ch < 16 * C::NKD) {
+                        if (C::VEC && a.dq.vec_ok && ch + 4 <= a.d) {
+                            u32x2_t pk;
+                            pk[0] = T::pack2(acc[qb][n][4 * bq] * a.scale, acc[qb][n][4 * bq + 1] * a.scale);
+                            pk[1] = T::pack2(acc[qb][n][4 * bq + 2] * a.scale, acc[qb][n][4 * bq + 3] * a.scale);
+                            *reinterpret_cast<u32x2_t *>(dqrow + ch) = pk;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (ch + e < a.d) dqrow[ch + e] = T::from_float(acc[qb][n][4 * bq + e] * a.scale);
+                        }
+                    } else if constexpr (C::NKR > 0) {
+                        const int cr = ch - 16 * C::NKD;
+                        if (C::VEC && a.dqb.vec_ok && cr + 4 <= a.r) {
+                            u32x2_t pk;
+                            pk[0] = T::pack2(acc[qb][n][4 * bq], acc[qb][n][4 * bq + 1]);
+                            pk[1] = T::pack2(acc[qb][n][4 * bq + 2], acc[qb][n][4 * bq + 3]);
+                            *reinterpret_cast<u32x2_t *>(dqbrow + cr) = pk;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (cr + e < a.r) dqbrow[cr + e] = T::from_float(acc[qb][n][4 * bq + e]);
+                        }
+                    }
+                }
+        }
+    }
+}
+
+template <class T, int NKD, int NKR, bool VEC, bool MASK>
+static hipError_t launch_dq_vec(const BwdArgs &a0, hipStream_t stream) {
+    typedef DqCfg<T, NKD, NKR, VEC, MASK> C;
+    BwdArgs a = a0;
+    a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
+    auto kern = bwd_dq_kernel<T, C>;
+    if (C::LDS_BYTES > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+    }
+    const int total = a.ntiles_m * a.B * a.H;
+    hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
+    return hipGetLastError();
+}
+
+template <class T, int NKD, int NKR>
+static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
+    const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+    if (a.mask.type)
+        return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
+    return vec ? launch_dq_vec<T, NKD, NKR, true, false>(a, stream) : launch_dq_vec<T, NKD, NKR, false, false>(a, stream);
+}
+
+template <class T, int NKD>
+static hipError_t launch_dq_r(const BwdArgs &a, hipStream_t stream) {
+    switch (nkr_of(a.r)) {
+    case 0: return launch_dq_cfg<T, NKD, 0>(a, stream);
+    case 1: return launch_dq_cfg<T, NKD, 1>(a, stream);
+    case 2: return launch_dq_cfg<T, NKD, 2>(a, stream);
+    case 4: return launch_dq_cfg<T, NKD, 4>(a, stream);
+    default: return launch_dq_cfg<T, NKD, 8>(a, stream);
+    }
+}
+
+// Compiled once per (element type, head-dim bucket), see Makefile.
+#define FB_CAT2(a, b) a##b
+#define FB_CAT(a, b) FB_CAT2(a, b)
+hipError_t FB_CAT(launch_bwd_dq_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
+    return launch_dq_r<FB_T, FB_NKD>(a, stream);
+}
+
+} // namespace fb

@@ -23,21 +23,18 @@ struct BwdArgs {
     MaskDesc mask;
     const float *lse; // (B, H, Lq)
     float *delta;     // (B, H, Lq)
-    float *dq_acc;    // (B*H, DQ_ROWS, Lq_pad) fp32: transposed partial sums of [dq | dq_bias]
-    int64_t lq_pad;   // row length of dq_acc
-    int dq_rows;      // rows of dq_acc per (batch, head)
-    int r_row0;       // first dq_bias row inside dq_acc (= d; rows [0, d) hold dq)
     int B, H, Lq, Lk, d, r;
     int causal;
     float scale;
-    int ntiles_n; // key tiles per (batch, head)
+    int ntiles_n; // key tiles per (batch, head), dk/dv kernel
+    int ntiles_m; // query tiles per (batch, head), dq kernel
 };
 
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.
 hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream);
-hipError_t launch_bwd_main(const BwdArgs &a, bool bf16, hipStream_t stream);
-hipError_t launch_bwd_finalize(const BwdArgs &a, bool bf16, hipStream_t stream);
+hipError_t launch_bwd_dkv(const BwdArgs &a, bool bf16, hipStream_t stream);
+hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream);
 
 // Padded sizes the dispatchers use: d is covered by 16-wide contraction steps of the
 // QK^T product (NKD of them) and the rank by NKR more; both rounded up to the next

@@ -114,9 +114,7 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
         dkb_full = torch.empty((p.B, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
         p.dq_bias, p.dk_bias = _tensor(dqb_full), _tensor(dkb_full)
     delta = torch.empty_like(lse)
-    nbytes = lib.fb_bwd_workspace_bytes(p)
-    workspace = torch.empty(nbytes // 4, device=q.device, dtype=torch.float32)
-    p.delta, p.workspace, p.workspace_bytes = delta.data_ptr(), workspace.data_ptr(), nbytes
+    p.delta = delta.data_ptr()
     with torch.cuda.device(q.device):
         _lib.check_status(lib.fb_bwd(p, _stream()))
     del keep

@@ -7,7 +7,7 @@
  * function it replaces.  Conventions shared by all of them:
  *
  *   - Nothing here allocates or frees device memory: every buffer, including scratch
- *     (lse, delta, the backward workspace), is owned by the caller, as in the reference where
+ *     (lse, delta), is owned by the caller, as in the reference where
  *     torch allocates o/lse/tmp/delta/dq_accum (flash_bias_triton.py:1145-1148, :1212-1219).
  *   - Launches are asynchronous on the given hipStream_t (passed as void*); no global
  *     mutable state, no autotuning side effects.
@@ -38,7 +38,7 @@ typedef enum fb_status {
     FB_ERR_DTYPE = -3,      /* only fp16 / bf16 inputs (flash_bias_triton.py:1108) */
     FB_ERR_STRIDE = -4,     /* stride would alias gradient rows / negative stride */
     FB_ERR_MASK = -5,       /* bad mask type / dtype */
-    FB_ERR_WORKSPACE = -6,  /* workspace missing or too small */
+    FB_ERR_RESERVED = -6,
     FB_ERR_ABI = -7,        /* fb_params.size does not match this library */
     FB_ERR_LAUNCH = -8,     /* HIP reported a launch error */
     FB_ERR_SCALE = -9       /* softmax scale not finite / not positive */
@@ -79,8 +79,6 @@ typedef struct fb_params {
     fb_tensor dq_bias, dk_bias; /* bwd out, full (B, L, H, r) shape: the caller reduces over
                                    broadcast dims */
     float *delta;               /* (B, H, Lq) fp32 scratch, written by the backward */
-    void *workspace;            /* fb_bwd_workspace_bytes() of device memory */
-    uint64_t workspace_bytes;
 } fb_params;
 
 /* Library / ABI version. */
@@ -98,24 +96,22 @@ int fb_check(const fb_params *p, int pass);
  * o = softmax(scale q k^T + q_bias k_bias^T + mask) v and lse. */
 int fb_fwd(const fb_params *p, void *stream);
 
-/* Bytes of device scratch the backward needs for these sizes (the reference's dq_accum /
- * dq_bias_accum, flash_bias_triton.py:1212-1219). */
-uint64_t fb_bwd_workspace_bytes(const fb_params *p);
-
 /* Replaces _flash_attn_backward (flash_bias_triton.py:1197-1342): runs the three phases
- * below in order on the stream. */
+ * below in order on the stream.  Unlike the reference there is no fp32 dq_accum buffer, no
+ * atomics and no final cast (:1212-1219, :1340-1342): dq and dq_bias are accumulated in
+ * registers by a query-stationary kernel and written once, so every gradient is
+ * bit-reproducible. */
 int fb_bwd(const fb_params *p, void *stream);
 
 /* The phases of fb_bwd, exported so that a harness can time them separately.
- *   fb_bwd_preprocess: delta = rowsum(o * dout) and zero the workspace
- *                      (_bwd_preprocess_do_o_dot, :358-400; init_to_zero, :872-879)
- *   fb_bwd_main:       recompute P from lse; dk, dv, dk_bias; dq / dq_bias partial sums
- *                      into the workspace (_bwd_kernel, :882-1097; :450-869)
- *   fb_bwd_finalize:   workspace -> dq (times scale) and dq_bias in the input dtype
- *                      (dq.copy_(dq_accum), :1340-1342) */
+ *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400)
+ *   fb_bwd_dkv:        recompute P from lse; dk, dv, dk_bias, one workgroup per key tile
+ *                      (_bwd_kernel / _bwd_kernel_one_col_block, :450-1097, minus dq)
+ *   fb_bwd_dq:         recompute P from lse; dq, dq_bias, one workgroup per query tile
+ *                      (the dq / dq_bias updates of :725-817) */
 int fb_bwd_preprocess(const fb_params *p, void *stream);
-int fb_bwd_main(const fb_params *p, void *stream);
-int fb_bwd_finalize(const fb_params *p, void *stream);
+int fb_bwd_dkv(const fb_params *p, void *stream);
+int fb_bwd_dq(const fb_params *p, void *stream);
 
 #ifdef __cplusplus
 }

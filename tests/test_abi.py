@@ -42,8 +42,6 @@ def _good(pass_=0):
         p.dout, p.dq, p.dk, p.dv = t(32), t(32), t(32), t(32)
         p.dq_bias, p.dk_bias = t(8), t(8)
         p.delta = fake
-        p.workspace = fake
-        p.workspace_bytes = _lib.load().fb_bwd_workspace_bytes(p)
     return p
 
 
@@ -52,14 +50,6 @@ def test_check_accepts_good_params():
     assert lib.fb_check(_good(0), 0) == 0
     assert lib.fb_check(_good(1), 1) == 0
     assert lib.fb_last_error() == b""
-
-
-def test_workspace_size_formula():
-    p = _good(1)
-    # (B*H) * (d + r) rows of round_up(Lq, 32) fp32 partial sums
-    assert _lib.load().fb_bwd_workspace_bytes(p) == 2 * 4 * (32 + 8) * 128 * 4
-    p.Lq = 100
-    assert _lib.load().fb_bwd_workspace_bytes(p) == 2 * 4 * (32 + 8) * 128 * 4
 
 
 @pytest.mark.parametrize("mutate,code", [
@@ -96,23 +86,20 @@ def test_check_rejects_forward(mutate, code):
     (lambda p: setattr(p, "delta", None), -1),
     (lambda p: setattr(p.dk, "stride_h", 0), -4),
     (lambda p: setattr(p.dk_bias, "stride_b", 0), -4),
-    (lambda p: setattr(p, "workspace", None), -6),
-    (lambda p: setattr(p, "workspace_bytes", 16), -6),
-    (lambda p: setattr(p, "workspace", 0x10004), -6),
 ])
 def test_check_rejects_backward(mutate, code):
     p = _good(1)
     mutate(p)
     lib = _lib.load()
     assert lib.fb_check(p, 1) == code
-    for fn in (lib.fb_bwd, lib.fb_bwd_preprocess, lib.fb_bwd_main, lib.fb_bwd_finalize):
+    for fn in (lib.fb_bwd, lib.fb_bwd_preprocess, lib.fb_bwd_dkv, lib.fb_bwd_dq):
         assert fn(p, None) == code
 
 
 def test_null_params():
     lib = _lib.load()
     assert lib.fb_check(None, 0) == -1
-    assert lib.fb_bwd_workspace_bytes(None) == 0
+    assert lib.fb_bwd(None, None) == -1
 
 
 def test_params_struct_matches_header_size():

@@ -163,8 +163,8 @@ def test_causal_structure_is_exact(gpu_device):
 
 
 def test_backward_reproducibility(gpu_device):
-    """dk, dv, dk_bias are accumulated in registers in a fixed order: bit-identical from run to
-    run.  dq / dq_bias go through fp32 atomics: equal up to summation order."""
+    """All five gradients are accumulated in registers in a fixed order (no atomics):
+    bit-identical from run to run."""
     dev = gpu_device
     ins = [t.to(dev).requires_grad_(True) for t in make_inputs(2, 700, 700, 4, 32, 8, torch.bfloat16, seed=6)[:5]]
     do = torch.randn(2, 700, 4, 32, device=dev, dtype=torch.bfloat16)
@@ -173,10 +173,8 @@ def test_backward_reproducibility(gpu_device):
         o = flash_bias_func(*ins, None, True, None)
         runs.append(torch.autograd.grad(o, ins, do))
     for other in runs[1:]:
-        for idx in (1, 2, 4):
+        for idx in range(5):
             assert torch.equal(runs[0][idx], other[idx])
-        for idx in (0, 3):
-            assert (runs[0][idx].float() - other[idx].float()).abs().max() <= 2e-2 * runs[0][idx].float().abs().max()
 
 
 # ------------------------------------------------------------------ named workloads (reduced)
