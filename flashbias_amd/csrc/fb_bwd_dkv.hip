@@ -30,7 +30,7 @@ struct DkvCfg {
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dK | dK_b]^T
-    static constexpr int KBW = (NK <= 4 && NDV <= 1) ? 2 : 1; // key blocks per wave
+    static constexpr int KBW = 1; // key blocks per wave
     static constexpr int BN = 32 * KBW * NWAVES;              // keys per workgroup
     static constexpr int QBLK = 2, BMQ = 32 * QBLK;           // queries per step
     static constexpr int DKP = 16 * NK + 8;  // sQ row (elements)

@@ -8,10 +8,9 @@
 // through double-buffered LDS.  With lane = query, register = key (transposed products):
 //
 //   S^T  = [K | K_b] [scale Q | Q_b]^T        A = key rows (LDS),        B = query registers
-//   dP^T = V dO^T - delta                     A = value rows (LDS),      B = dO registers,
-//                                             accumulator starts at -delta (a per-lane constant)
+//   dP^T = V dO^T                             A = value rows (LDS),      B = dO registers
 //   P^T  = exp(S^T - lse)                     lse is a per-lane scalar
-//   dS^T = P^T * dP^T
+//   dS^T = P^T * (dP^T - delta)               delta is a per-lane scalar
 //   [dQ | dQ_b]^T += [K | K_b]^T dS^T         A = transposed key tile (LDS), B = dS^T registers
 //
 // so dS^T goes from the accumulator layout straight into the next MFMA and [dQ | dQ_b]^T stays
@@ -169,8 +168,7 @@ bwd_dq_kernel(const BwdArgs a) {
     // ---- query-side operands, resident in registers
     u32x4_t qhi[C::QBLK][C::NKD], qlo[C::QBLK][C::NKD], qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
     u32x4_t dor[C::QBLK][C::NKD];
-    f32x16_t negd[C::QBLK]; // -delta of this lane's query in every element: start of the dP^T accumulator
-    float lse2[C::QBLK];
+    float negd[C::QBLK], lse2[C::QBLK]; // -delta and lse * log2(e) of this lane's queries
     f32x16_t acc[C::QBLK][C::MB];
 #pragma unroll
     for (int qb = 0; qb < C::QBLK; ++qb) {
@@ -189,9 +187,7 @@ bwd_dq_kernel(const BwdArgs a) {
         const bool ok = query < a.Lq;
         const int64_t sidx = (int64_t)bh * a.Lq + (ok ? query : a.Lq - 1);
         lse2[qb] = ok ? a.lse[sidx] * kLog2e : INFINITY; // rows past the end: P = exp2(-inf) = 0
-        const float nd = ok ? -a.delta[sidx] : 0.f;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) negd[qb][v] = nd;
+        negd[qb] = ok ? -a.delta[sidx] : 0.f;
 #pragma unroll
         for (int n = 0; n < C::MB; ++n)
 #pragma unroll
@@ -228,9 +224,9 @@ bwd_dq_kernel(const BwdArgs a) {
                 u32x4_t dsp[C::QBLK][2]; // dS^T, packed, per 16-key step
 #pragma unroll
                 for (int qb = 0; qb < C::QBLK; ++qb) {
-                    f32x16_t s, dp = negd[qb];
+                    f32x16_t s, dp;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+                    for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
 #pragma unroll
                     for (int t = 0; t < C::NK; ++t) {
                         if (t < C::NKD) {
@@ -261,7 +257,7 @@ bwd_dq_kernel(const BwdArgs a) {
                     for (int v = 0; v < 16; v += 2) {
                         const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[qb]));
                         const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[qb]));
-                        dsp[qb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
+                        dsp[qb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * (dp[v] + negd[qb]), p1 * (dp[v + 1] + negd[qb]));
                     }
                 }
                 // [dQ | dQ_b]^T += [K | K_b]^T dS^T over this block's 32 keys
