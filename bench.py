@@ -199,12 +199,23 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--report", action="store_true", help="table over all named workloads")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="before the run, copy a 256 MiB buffer 3 times (a plain copy kernel of known size, "
+                         "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no collective; (batch, head) pairs are "
                  "independent and would be split across GPUs with no exchange. Run with --gpus 1.")
     from flashbias_amd import _lib
     _lib.load()  # fail loudly if the HIP library is not built
+    if args.calibrate_copy:
+        import torch
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if args.report:
         report(args)
     else:
