@@ -98,8 +98,56 @@ __device__ __forceinline__ void dkv_load_step(DkvStage<C> &st, const BwdArgs &a,
     }
 }
 
+// Per-thread constants of the fast loader: a running global pointer per task (advanced by one
+// query step at a time) and the element offsets of the task's four rows.  Steps that lie
+// entirely inside the sequence are fetched with plain loads that nothing waits on until the
+// registers are written to LDS after the step's arithmetic.
 template <class C>
-__device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *stage, int tid) {
+struct DkvFast {
+    const uint16_t *ptr[C::PT];
+    uint32_t off[C::PT][4];
+    int64_t inc[C::PT];
+    bool ok[C::PT];
+
+    __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *qbase, const uint16_t *qbbase,
+                                         const uint16_t *dobase, int m0, int tid) {
+#pragma unroll
+        for (int i = 0; i < C::PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            int kind, quad, ch;
+            dkv_task<C>(task, kind, quad, ch);
+            const uint16_t *base = kind == 0 ? qbase : kind == 1 ? qbbase : dobase;
+            const int64_t ld = kind == 0 ? a.q.ss : kind == 1 ? a.qb.ss : a.dout.ss;
+            const int ncols = kind == 1 ? a.r : a.d;
+            ok[i] = task < C::TASKS && ch * 8 < ncols;
+            inc[i] = ok[i] ? ld * C::BMQ : 0;
+            ptr[i] = ok[i] ? base + (int64_t)m0 * ld + ch * 8 : qbase;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) off[i][j] = ok[i] ? (uint32_t)((quad * 4 + j) * ld) : 0u;
+        }
+    }
+
+    __device__ __forceinline__ void load(DkvStage<C> &st, const float *lse, const float *delta, int m0, int tid) {
+#pragma unroll
+        for (int i = 0; i < C::PT; ++i) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) st.x[i][j] = *reinterpret_cast<const u32x4_t *>(ptr[i] + off[i][j]);
+        }
+        if (tid < C::BMQ) {
+            st.lse2 = lse[m0 + tid];
+            st.negd = delta[m0 + tid];
+        }
+    }
+
+    __device__ __forceinline__ void advance() {
+#pragma unroll
+        for (int i = 0; i < C::PT; ++i) ptr[i] += inc[i];
+    }
+};
+
+template <class C>
+__device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *stage, int tid, const bool (&ok)[C::PT],
+                                               bool raw_stats) {
     uint16_t *sQ = stage, *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
     float *sStat = reinterpret_cast<float *>(sdOt + C::SDOT);
 #pragma unroll
@@ -107,7 +155,7 @@ __device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *
         const int task = tid + i * C::NTHREADS;
         int kind, quad, ch;
         dkv_task<C>(task, kind, quad, ch);
-        if (C::TASKS % C::NTHREADS == 0 || task < C::TASKS) {
+        if (ok[i]) { // chunks in the zero padding of the channel dim are never written (LDS cleared once)
             // row-major copy (A operand of S and dP) ...
             uint16_t *rm = kind == 2 ? sdO : sQ;
             const int ld = kind == 2 ? C::DOP : C::DKP;
@@ -128,9 +176,9 @@ __device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *
             }
         }
     }
-    if (tid < C::BMQ) {
-        sStat[tid] = st.lse2;
-        sStat[C::BMQ + tid] = st.negd;
+    if (tid < C::BMQ) { // the fast loader leaves lse and delta as read; convert here
+        sStat[tid] = raw_stats ? st.lse2 * kLog2e : st.lse2;
+        sStat[C::BMQ + tid] = raw_stats ? -st.negd : st.negd;
     }
 }
 
@@ -144,7 +192,7 @@ __device__ __forceinline__ float dkv_mask_at(const MaskDesc &m, const uint8_t *b
 }
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU))) void
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
 bwd_dkv_kernel(const BwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
@@ -207,10 +255,17 @@ bwd_dkv_kernel(const BwdArgs a) {
     const int step0 = a.causal ? n0 / C::BMQ : 0;
     const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
 
+    {   // clear both stages once: the zero padding of the channel dimension is never rewritten
+        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
+        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+    DkvFast<C> fast;
+    fast.init(a, qbase, qbbase, dobase, (step0 + 1) * C::BMQ, tid); // first prefetch is step0 + 1
     DkvStage<C> st;
     if (step0 < nsteps) {
         dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, step0 * C::BMQ, tid);
-        dkv_store_step<C>(st, stage0, tid);
+        dkv_store_step<C>(st, stage0, tid, fast.ok, false);
     }
     __syncthreads();
 
@@ -218,7 +273,15 @@ bwd_dkv_kernel(const BwdArgs a) {
         const int m0 = step * C::BMQ;
         const int cur = (step - step0) & 1;
         const bool more = step + 1 < nsteps;
-        if (more) dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, m0 + C::BMQ, tid);
+        // next step: plain in-flight loads if it lies inside the sequence, clamped loads otherwise
+        const bool next_fast = C::VEC && m0 + 2 * C::BMQ <= a.Lq;
+        if (more) {
+            if (next_fast)
+                fast.load(st, lse, delta, m0 + C::BMQ, tid);
+            else
+                dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, m0 + C::BMQ, tid);
+            fast.advance();
+        }
         const uint16_t *sQ = stage0 + cur * C::STAGE_ELEMS;
         const uint16_t *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
         const float *sStat = reinterpret_cast<const float *>(sdOt + C::SDOT);
@@ -304,7 +367,7 @@ bwd_dkv_kernel(const BwdArgs a) {
                 }
             }
         }
-        if (more) dkv_store_step<C>(st, stage0 + (cur ^ 1) * C::STAGE_ELEMS, tid);
+        if (more) dkv_store_step<C>(st, stage0 + (cur ^ 1) * C::STAGE_ELEMS, tid, fast.ok, next_fast);
         __syncthreads();
     }
 

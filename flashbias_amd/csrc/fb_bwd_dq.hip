@@ -90,7 +90,8 @@ struct DqLoader {
         }
     }
 
-    __device__ static __forceinline__ void store(const DqStage<C> &st, uint16_t *stage, int tid) {
+    __device__ static __forceinline__ void store(const DqStage<C> &st, uint16_t *stage, int tid,
+                                                 const bool (&kok)[C::K_PT], const bool (&vok)[C::V_PT]) {
         uint16_t *sK = stage, *sV = sK + C::SK, *sKt = sV + C::SV;
 #pragma unroll
         for (int i = 0; i < C::K_PT; ++i) {
@@ -98,7 +99,7 @@ struct DqLoader {
             int quad, ch;
             bool is_b;
             ktask(task, quad, ch, is_b);
-            if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS) {
+            if (kok[i]) {
                 const int col0 = (is_b ? 16 * C::NKD : 0) + ch * 8;
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -117,9 +118,62 @@ struct DqLoader {
 #pragma unroll
         for (int i = 0; i < C::V_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
-            if (C::V_TASKS % C::NTHREADS == 0 || task < C::V_TASKS)
-                *reinterpret_cast<u32x4_t *>(sV + (task % C::BN) * C::DVP + (task / C::BN) * 8) = st.v[i];
+            if (vok[i]) *reinterpret_cast<u32x4_t *>(sV + (task % C::BN) * C::DVP + (task / C::BN) * 8) = st.v[i];
         }
+    }
+};
+
+// Per-thread constants of the fast loader (tiles entirely inside the sequence): running global
+// pointers advanced by one key tile at a time, plain loads that stay in flight during the
+// tile's arithmetic.  Chunks that lie in the zero padding of the channel dimension are never
+// stored (the LDS buffers are cleared once).
+template <class C>
+struct DqFast {
+    const uint16_t *kptr[C::K_PT], *vptr[C::V_PT];
+    uint32_t koff[C::K_PT][4];
+    int64_t kinc[C::K_PT], vinc[C::V_PT];
+    bool kok[C::K_PT], vok[C::V_PT];
+
+    __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *kbase, const uint16_t *kbbase,
+                                         const uint16_t *vbase, int n0, int tid) {
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            int quad, ch;
+            bool is_b;
+            DqLoader<C>::ktask(task, quad, ch, is_b);
+            const uint16_t *base = is_b ? kbbase : kbase;
+            const int64_t ld = is_b ? a.kb.ss : a.k.ss;
+            kok[i] = task < C::K_TASKS && ch * 8 < (is_b ? a.r : a.d);
+            kinc[i] = kok[i] ? ld * C::BN : 0;
+            kptr[i] = kok[i] ? base + (int64_t)n0 * ld + ch * 8 : kbase;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) koff[i][j] = kok[i] ? (uint32_t)((quad * 4 + j) * ld) : 0u;
+        }
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) {
+            const int task = tid + i * C::NTHREADS;
+            const int row = task % C::BN, ch = task / C::BN;
+            vok[i] = task < C::V_TASKS && ch * 8 < a.d;
+            vinc[i] = vok[i] ? a.v.ss * C::BN : 0;
+            vptr[i] = vok[i] ? vbase + (int64_t)(n0 + row) * a.v.ss + ch * 8 : vbase;
+        }
+    }
+
+    __device__ __forceinline__ void load(DqStage<C> &st) const {
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) st.k[i][j] = *reinterpret_cast<const u32x4_t *>(kptr[i] + koff[i][j]);
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) st.v[i] = *reinterpret_cast<const u32x4_t *>(vptr[i]);
+    }
+
+    __device__ __forceinline__ void advance() {
+#pragma unroll
+        for (int i = 0; i < C::K_PT; ++i) kptr[i] += kinc[i];
+#pragma unroll
+        for (int i = 0; i < C::V_PT; ++i) vptr[i] += vinc[i];
     }
 };
 
@@ -198,16 +252,29 @@ bwd_dq_kernel(const BwdArgs a) {
     if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
     const int ntiles_k = (k_end + C::BN - 1) / C::BN;
 
+    {   // clear both LDS buffers once: the zero padding of the channel dimension is never rewritten
+        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
+        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+    DqFast<C> fast;
+    fast.init(a, kbase, kbbase, vbase, C::BN, tid); // the first prefetch is tile 1
     DqStage<C> st;
     DqLoader<C>::load(st, a, kbase, kbbase, vbase, 0, tid);
-    DqLoader<C>::store(st, stage0, tid);
+    DqLoader<C>::store(st, stage0, tid, fast.kok, fast.vok);
     __syncthreads();
 
     for (int it = 0; it < ntiles_k; ++it) {
         const int cur = it & 1;
         const int n0 = it * C::BN;
         const bool more = it + 1 < ntiles_k;
-        if (more) DqLoader<C>::load(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
+        if (more) {
+            if (C::VEC && n0 + 2 * C::BN <= a.Lk)
+                fast.load(st);
+            else
+                DqLoader<C>::load(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
+            fast.advance();
+        }
 
         const uint16_t *sK = stage0 + cur * C::STAGE, *sV = sK + C::SK, *sKt = sV + C::SV;
         const bool visible = !(a.causal && n0 > wq0 + 32 * C::QBLK - 1) && wq0 < a.Lq;
@@ -272,7 +339,7 @@ bwd_dq_kernel(const BwdArgs a) {
                     }
             }
         }
-        if (more) DqLoader<C>::store(st, stage0 + (cur ^ 1) * C::STAGE, tid);
+        if (more) DqLoader<C>::store(st, stage0 + (cur ^ 1) * C::STAGE, tid, fast.kok, fast.vok);
         __syncthreads();
     }
 
