@@ -164,32 +164,81 @@ def headline(args):
     print(json.dumps(out))
 
 
+def _sdpa_concat(w):
+    """The reference's pure-PyTorch FlashBias (flash_bias/attention_func.py:188-237): fused SDPA
+    over the concatenated features [q * scale, q_bias] / [k, k_bias] with scale 1."""
+    import torch
+    B, _, H, _ = w["q"].shape
+    qb = w["q_bias"].expand(B, -1, H, -1)
+    kb = w["k_bias"].expand(B, -1, H, -1)
+    qc = torch.cat([w["q"] * w["softmax_scale"], qb], -1)
+    kc = torch.cat([w["k"], kb], -1)
+    pad = (-qc.shape[-1]) % 8
+    if pad:
+        qc = torch.nn.functional.pad(qc, (0, pad))
+        kc = torch.nn.functional.pad(kc, (0, pad))
+    return torch.nn.functional.scaled_dot_product_attention(
+        qc.transpose(1, 2), kc.transpose(1, 2), w["v"].transpose(1, 2), is_causal=w["causal"], scale=1.0).transpose(1, 2)
+
+
+def _sdpa_dense(w, bias):
+    """SDPA with the materialised (B, H, Lq, Lk) bias as attn_mask (attention_func.py:150-185)."""
+    import torch
+    return torch.nn.functional.scaled_dot_product_attention(
+        w["q"].transpose(1, 2), w["k"].transpose(1, 2), w["v"].transpose(1, 2), attn_mask=bias,
+        scale=w["softmax_scale"]).transpose(1, 2)
+
+
+def _time_torch(make_out, leaves, do, steps, warmup):
+    """fwd and fwd+bwd milliseconds of a torch provider."""
+    import torch
+    fwd = _time_events(lambda: make_out(), steps, warmup)
+
+    def fb():
+        torch.autograd.grad(make_out(), leaves, do)
+    return fwd, _time_events(fb, steps, warmup)
+
+
 def report(args):
-    """fwd / fwd+bwd milliseconds and TFLOP/s over the named workloads (informational)."""
+    """fwd / fwd+bwd milliseconds and TFLOP/s over the named workloads, next to what PyTorch-ROCm
+    offers for the same math (SDPA on concatenated features; SDPA with a dense bias where the
+    N x N bias fits comfortably).  Informational, not part of the one-line contract."""
     import torch
     from flashbias_amd import workloads
     dev = torch.device("cuda:0")
     rows = []
-    cases = [(f"sweep L={L}", lambda L=L: workloads.sweep(L)) for L in workloads.SWEEP_LENGTHS]
-    cases += [(f"alibi causal L={L}", lambda L=L: workloads.alibi(L)) for L in (2048, 4096, 8192)]
-    cases += [("swin 4096x256 r16", lambda: workloads.swin()), ("pde N=32768 r5", lambda: workloads.pde()),
-              ("pairformer 768 r32", lambda: workloads.pairformer())]
-    for name, make in cases:
+    cases = [(f"sweep L={L}", lambda L=L: workloads.sweep(L), True) for L in workloads.SWEEP_LENGTHS]
+    cases += [(f"alibi causal L={L}", lambda L=L: workloads.alibi(L), False) for L in (2048, 4096, 8192)]
+    cases += [("swin 4096x256 r16", lambda: workloads.swin(), False), ("pde N=32768 r5", lambda: workloads.pde(), False),
+              ("pairformer 768 r32", lambda: workloads.pairformer(), False)]
+    for name, make, dense in cases:
         w = _to_dev(make(), dev)
         B, Lq, H, d = w["q"].shape
         r = w["q_bias"].shape[-1]
         f_fwd, f_bwd = workloads.flops(B, H, Lq, w["k"].shape[1], d, r, w["causal"])
         phases, keep = _phase_timers(w, dev)
         ms = {n: _time_events(fn, args.steps, args.warmup) for n, fn in phases.items()}
-        bwd = ms["fb_bwd_preprocess"] + ms["fb_bwd_dkv"] + ms["fb_bwd_dq"]
-        rows.append((name, ms["fb_fwd"], f_fwd / ms["fb_fwd"] / 1e9, ms["fb_fwd"] + bwd,
-                     (f_fwd + f_bwd) / (ms["fb_fwd"] + bwd) / 1e9))
-        del keep, w
+        ours_fwd = ms["fb_fwd"]
+        ours_fb = ours_fwd + ms["fb_bwd_preprocess"] + ms["fb_bwd_dkv"] + ms["fb_bwd_dq"]
+        del keep
+        leaves = [w[n].requires_grad_(True) for n in ("q", "k", "v", "q_bias", "k_bias")]
+        cat_fwd, cat_fb = _time_torch(lambda: _sdpa_concat(w), leaves, w["do"], args.steps, args.warmup)
+        den_fwd = den_fb = float("nan")
+        if dense:
+            with torch.no_grad():
+                bias = (w["q_bias"].permute(0, 2, 1, 3) @ w["k_bias"].permute(0, 2, 3, 1)).contiguous()
+            den_fwd, den_fb = _time_torch(lambda: _sdpa_dense(w, bias), leaves[:3], w["do"], args.steps, args.warmup)
+            del bias
+        rows.append((name, ours_fwd, f_fwd / ours_fwd / 1e9, ours_fb, (f_fwd + f_bwd) / ours_fb / 1e9, cat_fwd, cat_fb,
+                     den_fwd, den_fb))
+        del w, leaves
         torch.cuda.empty_cache()
-    print("| workload | fwd ms | fwd TFLOP/s | fwd+bwd ms | fwd+bwd TFLOP/s | % bf16 peak |")
-    print("|---|---|---|---|---|---|")
-    for name, a, b, c, d_ in rows:
-        print(f"| {name} | {a:.3f} | {b:.1f} | {c:.3f} | {d_:.1f} | {100 * d_ / PEAK_BF16_TFLOPS:.1f} |")
+    print("| workload | fwd ms | fwd TFLOP/s | fwd+bwd ms | fwd+bwd TFLOP/s | % bf16 peak | SDPA-concat fwd / fwd+bwd ms "
+          "| SDPA dense-bias fwd / fwd+bwd ms |")
+    print("|---|---|---|---|---|---|---|---|")
+    for name, a, b, c, d_, e, f, g, h in rows:
+        print(f"| {name} | {a:.3f} | {b:.1f} | {c:.3f} | {d_:.1f} | {100 * d_ / PEAK_BF16_TFLOPS:.1f} | {e:.3f} / {f:.3f} "
+              f"| {g:.3f} / {h:.3f} |")
 
 
 def main():

@@ -60,6 +60,12 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
         assert q_bias.is_cuda and k_bias.is_cuda
         rank = q_bias.shape[-1]
         assert k_bias.shape[-1] == rank
+        if rank % 8:
+            # zero columns change nothing in q_bias k_bias^T; a multiple of 8 makes the rows 16-byte
+            # aligned, which selects the kernels with vector loads (ALiBi r=2, distance bias r=5)
+            pad = (0, 8 - rank % 8)
+            q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
+            rank = q_bias.shape[-1]
         # stride-0 broadcast over batch / heads (:1135-1136)
         qbe = q_bias.expand(batch, seqlen_q, nheads, rank)
         kbe = k_bias.expand(batch, seqlen_k, nheads, rank)
@@ -120,8 +126,9 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     del keep
     dq_bias = dk_bias = None
     if q_bias is not None:
-        dq_bias = _reduce_like(dqb_full, q_bias)
-        dk_bias = _reduce_like(dkb_full, k_bias)
+        r = q_bias.shape[-1]  # the kernels may have run on zero-padded factors
+        dq_bias = _reduce_like(dqb_full[..., :r], q_bias)
+        dk_bias = _reduce_like(dkb_full[..., :r], k_bias)
     return dq, dk, dv, dq_bias, dk_bias
 
 
@@ -129,8 +136,8 @@ def _reduce_like(full, ref):
     """Sum a full (B, L, H, r) gradient over the dims in which ``ref`` was broadcast."""
     dims = [i for i in (0, 2) if ref.shape[i] == 1 and full.shape[i] != 1]
     if dims:
-        full = full.sum(dim=dims, keepdim=True, dtype=torch.float32).to(ref.dtype)
-    return full
+        return full.sum(dim=dims, keepdim=True, dtype=torch.float32).to(ref.dtype)
+    return full if full.is_contiguous() else full.contiguous()
 
 
 class FlashBiasFunc(torch.autograd.Function):

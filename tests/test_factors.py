@@ -1,0 +1,84 @@
+"""CPU tests of the factor builders and workload generators (closed forms and invariants)."""
+import math
+
+import torch
+
+from flashbias_amd import factors, workloads
+
+
+def _dense(q_bias, k_bias):
+    return q_bias.permute(0, 2, 1, 3).double() @ k_bias.permute(0, 2, 3, 1).double()
+
+
+def test_alibi_slopes_and_factors_closed_form():
+    """m_h = 2^(-8 (h+1) / H) (attention_with_alibi_bias.py:8-15); bias_ij = -m_h (i - j)."""
+    for H in (4, 8, 50):
+        m = factors.alibi_slopes(H).double()
+        ref = torch.tensor([(2.0 ** 8) ** (-(h + 1) / H) for h in range(H)], dtype=torch.float64)
+        assert torch.allclose(m, ref, rtol=1e-6)
+    qb, kb = factors.alibi_factors(33, 47, 8)
+    assert qb.shape == (1, 33, 8, 2) and kb.shape == (1, 47, 8, 2)
+    i, j = torch.arange(33.0).double(), torch.arange(47.0).double()
+    want = -factors.alibi_slopes(8).double()[:, None, None] * (i[:, None] - j[None, :])
+    assert torch.allclose(_dense(qb, kb)[0], want, atol=1e-5)
+
+
+def test_distance_factors_identity():
+    """-alpha |x_i - x_j|^2 = [-alpha|x_i|^2, -alpha, 2 alpha x_i] . [1, |x_j|^2, x_j], exact rank D+2."""
+    g = torch.Generator().manual_seed(0)
+    xq = torch.rand(2, 40, 3, generator=g, dtype=torch.float64)
+    xk = torch.rand(2, 50, 3, generator=g, dtype=torch.float64)
+    qb, kb = factors.distance_factors(xq, xk, 10.0, torch.float64)
+    assert qb.shape == (2, 40, 1, 5) and kb.shape == (2, 50, 1, 5)
+    want = -10.0 * torch.cdist(xq, xk) ** 2
+    assert torch.allclose(_dense(qb, kb)[:, 0], want, atol=1e-12)
+
+
+def test_svd_factors_are_eckart_young_optimal():
+    g = torch.Generator().manual_seed(1)
+    bias = torch.randn(3, 24, 24, generator=g, dtype=torch.float64)
+    qb, kb, rel = factors.svd_factors(bias, 6, torch.float64)
+    rec = _dense(qb, kb)[0]
+    s = torch.linalg.svdvals(bias)
+    tail = (s[:, 6:] ** 2).sum(-1).sqrt()
+    assert torch.allclose((rec - bias).flatten(1).norm(dim=1), tail, rtol=1e-9)
+    assert torch.allclose(rel.double(), tail / bias.flatten(1).norm(dim=1), rtol=1e-5)
+    full_q, full_k, rel0 = factors.svd_factors(bias, 24, torch.float64)
+    assert torch.allclose(_dense(full_q, full_k)[0], bias, atol=1e-10) and rel0.max() < 1e-6
+
+
+def test_swin_table_structure():
+    """Relative-position bias: depends on (dy, dx) only, lies in (0, 16), low effective rank."""
+    t = factors.swin_v2_bias_table(8, 4, seed=3)
+    assert t.shape == (4, 64, 64) and t.min() > 0 and t.max() < 16
+    idx = lambda y, x: y * 8 + x
+    assert torch.equal(t[:, idx(2, 3), idx(1, 1)], t[:, idx(5, 6), idx(4, 4)])  # same (dy, dx) = (1, 2)
+    _, _, rel = factors.svd_factors(t, 16)
+    assert rel.max() < 0.05
+
+
+def test_workloads_are_seeded_and_shaped():
+    a, b = workloads.sweep(256, seed=5), workloads.sweep(256, seed=5)
+    assert all(torch.equal(a[n], b[n]) for n in ("q", "k", "v", "q_bias", "k_bias", "do"))
+    assert a["q"].shape == (2, 256, 4, 32) and a["q_bias"].shape == (2, 256, 4, 8) and a["q"].dtype == torch.bfloat16
+    assert abs(a["q_bias"].float().std().item() - 1 / math.sqrt(8)) < 0.02
+    w = workloads.alibi(128, H=6)
+    assert w["causal"] and w["q_bias"].shape == (1, 128, 6, 2)
+    w = workloads.swin(windows=3, window=4, H=2, r=4)
+    assert w["q"].shape == (3, 16, 2, 32) and w["q_bias"].shape == (1, 16, 2, 4)
+    w = workloads.pde(N=64, H=2)
+    assert w["q_bias"].shape == (1, 64, 1, 5)
+    w = workloads.pairformer(N=16, H=2, r=8)
+    assert w["q"].shape == (16, 16, 2, 32) and w["k_bias"].shape == (1, 16, 2, 8)
+
+
+def test_flop_formulas():
+    fwd, bwd = workloads.flops(2, 4, 16384, 16384, 32, 8)
+    assert fwd == 2 * 2 * 4 * 16384 ** 2 * 72 and bwd == 2 * 2 * 4 * 16384 ** 2 * 184
+    assert abs(fwd + bwd - 1.0995e12) < 1e9
+    cf, _ = workloads.flops(1, 1, 100, 100, 32, 8, causal=True)
+    assert cf == 2 * 5050 * 72
+    rect, _ = workloads.flops(1, 1, 5, 3, 4, 0, causal=True)
+    assert rect == 2 * (1 + 2 + 3 + 3 + 3) * 8
+    rf, rfb = workloads.reference_formula_flops(2, 4, 16384, 32)
+    assert abs(rf - 2.770e11) < 1e8 and rfb == 3 * rf
