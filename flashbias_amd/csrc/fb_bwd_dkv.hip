@@ -44,7 +44,11 @@ struct DkvCfg {
     static constexpr int QUADS = BMQ / 4;
     static constexpr int TASKS = QUADS * (CQ + CR + CO);
     static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
+#ifdef FB_W3
+    static constexpr int WAVES_EU = 3;
+#else
     static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 2 : 1;
+#endif
 };
 
 template <class C>
@@ -192,7 +196,7 @@ __device__ __forceinline__ float dkv_mask_at(const MaskDesc &m, const uint8_t *b
 }
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::WAVES_EU == 3 ? 0 : 1)))) void
 bwd_dkv_kernel(const BwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);

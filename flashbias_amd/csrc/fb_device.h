@@ -137,6 +137,15 @@ __device__ __forceinline__ int xcd_remap(int wg, int total) {
     return (wg % kXcd) * (total / kXcd) + wg / kXcd;
 }
 
+// max(x of this lane, x of lane ^ 32): v_permlane32_swap exchanges the upper half of its first
+// operand with the lower half of its second, so both copies end up holding one half's value in
+// every lane.  A VALU exchange: no trip through the LDS crossbar.
+__device__ __forceinline__ float half_wave_max(float x) {
+    float lo = x, hi = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
+    return fmaxf(lo, hi);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // scale * x for the eight 16-bit values of a chunk, as hi + lo parts in the same 16-bit type

@@ -1,8 +1,9 @@
 // Forward FlashBias attention for gfx950:  o = softmax(scale q k^T + q_b k_b^T + mask) v, lse.
 // Replaces _fwd_kernel of the reference (flash_bias/flash_bias_triton.py:62-355).
 //
-// One workgroup (4 waves) owns BM = 128 consecutive queries of one (batch, head); each wave
-// owns 32 of them.  Keys are streamed in tiles of BN = 64 through double-buffered LDS.
+// One workgroup (4 waves) owns BM = 128 or 256 consecutive queries of one (batch, head); each
+// wave owns one or two blocks of 32 of them.  Keys are streamed in tiles of BN = 64 or 128
+// through double-buffered LDS.
 // Everything is computed transposed so that a lane owns one query:
 //
 //   S^T (keys x queries) = [K | K_b] [scale Q | Q_b]^T     A = key tile from LDS, B = query regs
@@ -35,9 +36,17 @@ struct FwdCfg {
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
-    static constexpr int BM = NWAVES * 32;
-    static constexpr int KBLK = 2, BN = 32 * KBLK;
+    // query blocks (of 32) per wave: two where the registers allow, so that every key / value
+    // fragment read from LDS feeds two blocks and two waves per SIMD carry four softmax streams
+    static constexpr int QB = (NKD_ + NKR_ <= 3 && NDV_ == 1 && VEC_ && !MASK_) ? 2 : 1;
+    static constexpr int BM = NWAVES * 32 * QB;
     static constexpr int NK = NKD + NKR;
+    // A wave computes KBLK * 32 keys at a time; an LDS tile (one barrier) holds SUBS such groups.
+    static constexpr int KBLK = 2, BSUB = 32 * KBLK;
+    // two groups per tile where three workgroups of that size still fit the 160 KB of a CU
+    static constexpr int LDS2 = 2 * 2 * (2 * BSUB * (16 * NK + 8) + 32 * NDV_ * (2 * BSUB + 8));
+    static constexpr int SUBS = (NK <= 4 && NDV_ <= 2 && 3 * LDS2 <= 160 * 1024) ? 2 : 1;
+    static constexpr int BN = BSUB * SUBS;
     static constexpr int DKP = 16 * NK + 8; // LDS row of [K | K_b], elements (16 B of padding)
     static constexpr int DV = 32 * NDV;
     static constexpr int BNP = BN + 8; // LDS row of V^T
@@ -51,7 +60,11 @@ struct FwdCfg {
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int KB_PT = (KB_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
-    static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 3 : 2;
+    static constexpr int WAVES_EU = QB == 2 ? 2 : (NK <= 4 && NDV <= 2) ? 3 : 2;
+    // LDS fragments requested ahead of their use: all key steps of a group when they are few,
+    // and the V^T fragments of a group when the head dimension is one MFMA block
+    static constexpr int KPRE = NK <= 4 ? NK : 0;
+    static constexpr bool VPRE = NDV == 1;
 };
 
 template <class C>
@@ -208,7 +221,8 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     uint16_t *sKbuf = reinterpret_cast<uint16_t *>(smem);
     uint16_t *sVbuf = sKbuf + 2 * C::SK_ELEMS;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // scalar: branches on it are uniform
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_m * a.B * a.H;
@@ -218,8 +232,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
-    const int wq0 = m0 + wave * 32; // first query of this wave
-    const int query = wq0 + c;
+    const int wq0 = m0 + wave * (32 * C::QB); // first query of this wave
 
     const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
     const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
@@ -234,25 +247,32 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
-    // ---- query operand, resident in registers for the whole key loop
-    u32x4_t qhi[C::NKD], qlo[C::NKD], qbr[C::NKR > 0 ? C::NKR : 1];
+    // ---- query operands, resident in registers for the whole key loop
+    u32x4_t qhi[C::QB][C::NKD], qlo[C::QB][C::NKD], qbr[C::QB][C::NKR > 0 ? C::NKR : 1];
+    f32x16_t acc_o[C::QB][C::NDV];
+    float m_ref[C::QB]; // reference of the exponentials (natural units), lags the true row max
+    float m2[C::QB];    // m_ref * log2(e), 0 while the row has seen no finite score
+    float l_run[C::QB]; // per-lane partial row sum (the two lanes of a query are added at the end)
 #pragma unroll
-    for (int t = 0; t < C::NKD; ++t)
-        split_scaled<T>(load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d), a.scale, qhi[t], qlo[t]);
-    if constexpr (C::NKR > 0) {
+    for (int qb = 0; qb < C::QB; ++qb) {
+        const int query = wq0 + 32 * qb + c;
 #pragma unroll
-        for (int t = 0; t < C::NKR; ++t)
-            qbr[t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * t + 8 * g, a.r);
+        for (int t = 0; t < C::NKD; ++t)
+            split_scaled<T>(load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d), a.scale, qhi[qb][t],
+                            qlo[qb][t]);
+        if constexpr (C::NKR > 0) {
+#pragma unroll
+            for (int t = 0; t < C::NKR; ++t)
+                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * t + 8 * g, a.r);
+        }
+#pragma unroll
+        for (int n = 0; n < C::NDV; ++n)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc_o[qb][n][v] = 0.f;
+        m_ref[qb] = -INFINITY;
+        m2[qb] = 0.f;
+        l_run[qb] = 0.f;
     }
-
-    f32x16_t acc_o[C::NDV];
-#pragma unroll
-    for (int n = 0; n < C::NDV; ++n)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc_o[n][v] = 0.f;
-    float m_ref = -INFINITY; // reference of the exponentials (natural units), lags the true row max
-    float m2 = 0.f;          // m_ref * log2(e), 0 while the row has seen no finite score
-    float l_run = 0.f;       // per-lane partial row sum (the two lanes of a query are added at the end)
     constexpr float kLagNat = 8.0f * kLn2; // let the row max run ahead of m_ref by up to 2^8
 
     // causal: tiles past the last query of this workgroup are never visible (:202)
@@ -287,88 +307,123 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 
         const uint16_t *sK = sKbuf + cur * C::SK_ELEMS;
         const uint16_t *sVt = sVbuf + cur * C::SV_ELEMS;
-        const bool visible = !(a.causal && n0 > wq0 + 31) && wq0 < a.Lq;
-        if (visible) {
-            // ---- S^T = [K | K_b] [scale Q | Q_b]^T
-            f32x16_t s[C::KBLK];
-#pragma unroll
-            for (int kb = 0; kb < C::KBLK; ++kb) {
-                f32x16_t acc;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = 0.f;
-#pragma unroll
-                for (int t = 0; t < C::NK; ++t) {
-                    const u32x4_t ka =
-                        *reinterpret_cast<const u32x4_t *>(sK + (kb * 32 + c) * C::DKP + 16 * t + 8 * g);
-                    if (t < C::NKD) {
-                        acc = T::mfma(ka, qhi[t], acc);
-                        acc = T::mfma(ka, qlo[t], acc);
-                    } else {
-                        acc = T::mfma(ka, qbr[t - C::NKD], acc);
-                    }
-                }
-                s[kb] = acc;
-            }
-            // ---- additive mask, then -inf for keys past the end and causal-hidden pairs
-            if constexpr (C::MASK) {
-#pragma unroll
-                for (int kb = 0; kb < C::KBLK; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
-                        s[kb][v] += mask_at<T>(a.mask, mbase, query, key, a.Lq, a.Lk);
-                    }
-            }
-            const bool ragged = n0 + C::BN > a.Lk;
-            const bool diag = a.causal && (n0 + C::BN - 1 > wq0);
-            if (ragged || diag) {
-#pragma unroll
-                for (int kb = 0; kb < C::KBLK; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
-                        if (key >= a.Lk || (a.causal && key > query)) s[kb][v] = -INFINITY;
-                    }
-            }
-            // ---- online softmax, one query per lane (two lanes share a query)
-            float mx = s[0][0];
+#pragma nounroll
+        for (int sub = 0; sub < C::SUBS; ++sub) {
+            const int ns = n0 + sub * C::BSUB;
+            // the group is hidden from every query of this wave: so are all later ones
+            if ((a.causal && ns > wq0 + 32 * C::QB - 1) || wq0 >= a.Lq || ns >= k_end) break;
+            // all key fragments of the group are requested before the first MFMA (one LDS wait)
+            // and serve every query block of the wave
+            u32x4_t ka[C::KBLK][C::KPRE > 0 ? C::KPRE : 1];
 #pragma unroll
             for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
-                for (int v = (kb == 0 ? 1 : 0); v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const bool grow = mx > m_ref + kLagNat; // also true for the first finite score of a row
-            if (__any(grow)) {
-                const float m_new = grow ? mx : m_ref;
-                const float alpha = grow ? fast_exp2((m_ref - m_new) * kLog2e) : 1.f; // exp2(-inf) = 0
-                l_run *= alpha;
+                for (int t = 0; t < C::KPRE; ++t)
+                    ka[kb][t] = *reinterpret_cast<const u32x4_t *>(sK + (sub * C::BSUB + kb * 32 + c) * C::DKP +
+                                                                   16 * t + 8 * g);
+            // the V^T fragments travel from LDS while the first row maximum is formed
+            u32x4_t va[C::VPRE ? C::KBLK * 2 : 1];
+            if constexpr (C::VPRE) {
 #pragma unroll
-                for (int n = 0; n < C::NDV; ++n)
+                for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc_o[n][v] *= alpha;
-                m_ref = m_new;
-                m2 = (m_ref == -INFINITY) ? 0.f : m_ref * kLog2e;
+                    for (int t = 0; t < 2; ++t)
+                        va[kb * 2 + t] = *reinterpret_cast<const u32x4_t *>(sVt + c * C::BNP + sub * C::BSUB + kb * 32 +
+                                                                            16 * t + 8 * g);
             }
-            // ---- P^T = exp(S^T - m_ref), row sums, O^T += V^T P^T
 #pragma unroll
-            for (int kb = 0; kb < C::KBLK; ++kb)
+            for (int qb = 0; qb < C::QB; ++qb) {
+                const int bq0 = wq0 + 32 * qb; // first query of the block
+                const int query = bq0 + c;
+                // wave-uniform skip of a block the whole group is hidden from (it also keeps the
+                // instruction streams of the two blocks apart, which the register allocation needs)
+                if (C::QB > 1 && a.causal && ns > bq0 + 31) continue;
+                // ---- S^T = [K | K_b] [scale Q | Q_b]^T
+                f32x16_t s[C::KBLK];
 #pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    u32x4_t pb;
+                for (int kb = 0; kb < C::KBLK; ++kb) {
+                    f32x16_t acc;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float p0 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e], kLog2e, -m2));
-                        const float p1 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e + 1], kLog2e, -m2));
-                        pb[e] = T::pack2(p0, p1);
-                        l_run = T::dot2_ones(pb[e], l_run);
+                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+                    for (int t = 0; t < C::NK; ++t) {
+                        const u32x4_t kf = t < C::KPRE ? ka[kb][t < C::KPRE ? t : 0]
+                                                       : *reinterpret_cast<const u32x4_t *>(
+                                                             sK + (sub * C::BSUB + kb * 32 + c) * C::DKP + 16 * t + 8 * g);
+                        if (t < C::NKD) {
+                            acc = T::mfma(kf, qhi[qb][t], acc);
+                            acc = T::mfma(kf, qlo[qb][t], acc);
+                        } else {
+                            acc = T::mfma(kf, qbr[qb][t - C::NKD], acc);
+                        }
                     }
-#pragma unroll
-                    for (int n = 0; n < C::NDV; ++n) {
-                        const u32x4_t va = *reinterpret_cast<const u32x4_t *>(
-                            sVt + (32 * n + c) * C::BNP + kb * 32 + 16 * t + 8 * g);
-                        acc_o[n] = T::mfma(va, pb, acc_o[n]);
-                    }
+                    s[kb] = acc;
                 }
+                // ---- additive mask, then -inf for keys past the end and causal-hidden pairs
+                if constexpr (C::MASK) {
+#pragma unroll
+                    for (int kb = 0; kb < C::KBLK; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = ns + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            s[kb][v] += mask_at<T>(a.mask, mbase, query, key, a.Lq, a.Lk);
+                        }
+                }
+                const bool ragged = ns + C::BSUB > a.Lk;
+                const bool diag = a.causal && (ns + C::BSUB - 1 > bq0);
+                if (ragged || diag) {
+#pragma unroll
+                    for (int kb = 0; kb < C::KBLK; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = ns + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            if (key >= a.Lk || (a.causal && key > query)) s[kb][v] = -INFINITY;
+                        }
+                }
+                // ---- online softmax, one query per lane (two lanes share a query)
+                float mx = s[0][0];
+#pragma unroll
+                for (int kb = 0; kb < C::KBLK; ++kb)
+#pragma unroll
+                    for (int v = (kb == 0 ? 1 : 0); v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
+                mx = half_wave_max(mx);
+                const bool grow = mx > m_ref[qb] + kLagNat; // also true for the first finite score of a row
+                if (__any(grow)) {
+                    const float m_new = grow ? mx : m_ref[qb];
+                    const float alpha = grow ? fast_exp2((m_ref[qb] - m_new) * kLog2e) : 1.f; // exp2(-inf) = 0
+                    l_run[qb] *= alpha;
+#pragma unroll
+                    for (int n = 0; n < C::NDV; ++n)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc_o[qb][n][v] *= alpha;
+                    m_ref[qb] = m_new;
+                    m2[qb] = (m_new == -INFINITY) ? 0.f : m_new * kLog2e;
+                }
+                // ---- P^T = exp(S^T - m_ref), row sums (of the fp32 values, :271), O^T += V^T P^T
+#pragma unroll
+                for (int kb = 0; kb < C::KBLK; ++kb)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        u32x4_t pb;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const float p0 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e], kLog2e, -m2[qb]));
+                            const float p1 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e + 1], kLog2e, -m2[qb]));
+                            pb[e] = T::pack2(p0, p1);
+                            l_run[qb] += p0 + p1;
+                        }
+                        if constexpr (C::VPRE) {
+                            acc_o[qb][0] = T::mfma(va[kb * 2 + t], pb, acc_o[qb][0]);
+                        } else {
+#pragma unroll
+                            for (int n = 0; n < C::NDV; ++n) {
+                                const u32x4_t vf = *reinterpret_cast<const u32x4_t *>(
+                                    sVt + (32 * n + c) * C::BNP + sub * C::BSUB + kb * 32 + 16 * t + 8 * g);
+                                acc_o[qb][n] = T::mfma(vf, pb, acc_o[qb][n]);
+                            }
+                        }
+                    }
+            }
         }
         if (more) ld.store(st, sKbuf + (cur ^ 1) * C::SK_ELEMS, sVbuf + (cur ^ 1) * C::SV_ELEMS);
         __syncthreads();
@@ -376,27 +431,31 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 
     // ---- epilogue: o = acc / l, lse = m_ref + ln(l)
     uint16_t *obase = const_cast<uint16_t *>(a.o.ptr) + b * a.o.sb + h * a.o.sh;
-    const float l = l_run + __shfl_xor(l_run, 32, 64);
-    const float inv = 1.f / l;
-    if (query < a.Lq) {
-        if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref + __builtin_amdgcn_logf(l) * kLn2;
-        uint16_t *orow = obase + (int64_t)query * a.o.ss;
 #pragma unroll
-        for (int n = 0; n < C::NDV; ++n)
+    for (int qb = 0; qb < C::QB; ++qb) {
+        const int query = wq0 + 32 * qb + c;
+        const float l = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
+        const float inv = 1.f / l;
+        if (query < a.Lq) {
+            if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref[qb] + __builtin_amdgcn_logf(l) * kLn2;
+            uint16_t *orow = obase + (int64_t)query * a.o.ss;
 #pragma unroll
-            for (int bq = 0; bq < 4; ++bq) {
-                const int ch = 32 * n + 8 * bq + 4 * g;
-                if (C::VEC && ch + 4 <= a.d) {
-                    u32x2_t pk;
-                    pk[0] = T::pack2(acc_o[n][4 * bq] * inv, acc_o[n][4 * bq + 1] * inv);
-                    pk[1] = T::pack2(acc_o[n][4 * bq + 2] * inv, acc_o[n][4 * bq + 3] * inv);
-                    *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
-                } else {
+            for (int n = 0; n < C::NDV; ++n)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (ch + e < a.d) orow[ch + e] = T::from_float(acc_o[n][4 * bq + e] * inv);
+                for (int bq = 0; bq < 4; ++bq) {
+                    const int ch = 32 * n + 8 * bq + 4 * g;
+                    if (C::VEC && ch + 4 <= a.d) {
+                        u32x2_t pk;
+                        pk[0] = T::pack2(acc_o[qb][n][4 * bq] * inv, acc_o[qb][n][4 * bq + 1] * inv);
+                        pk[1] = T::pack2(acc_o[qb][n][4 * bq + 2] * inv, acc_o[qb][n][4 * bq + 3] * inv);
+                        *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (ch + e < a.d) orow[ch + e] = T::from_float(acc_o[qb][n][4 * bq + e] * inv);
+                    }
                 }
-            }
+        }
     }
 }
 
