@@ -11,7 +11,7 @@
 //   dP^T = V dO^T                             A = value rows (LDS),      B = dO registers
 //   P^T  = exp(S^T - lse)                     lse is a per-lane scalar
 //   dS^T = P^T * (dP^T - delta)               delta is a per-lane scalar
-//   [dQ | dQ_b]^T += [K | K_b]^T dS^T         A = transposed key tile (LDS), B = dS^T registers
+//   [dQ | dQ_b]^T += [K | K_b]^T dS^T         A = key tile read column-wise (LDS), B = dS^T registers
 //
 // so dS^T goes from the accumulator layout straight into the next MFMA and [dQ | dQ_b]^T stays
 // in registers for the whole key loop: each output element is written exactly once, in a fixed
@@ -35,17 +35,16 @@ struct DqCfg {
 #endif
     static constexpr int BM = NWAVES * QBLK * 32;
     static constexpr int KBLK = 2, BN = 32 * KBLK;
-    static constexpr int DKP = 16 * NK + 8;  // sK row: [K | K_b] of one key
+    // sK row: [K | K_b] of one key in ROWCH swizzled 16-byte chunks; the one copy is read
+    // row-wise for S^T and column-wise for [dQ | dQ_b]^T
+    static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
     static constexpr int DVP = 16 * NKD + 8; // sV row: V of one key
-    static constexpr int BNP = BN + 8;       // sKt row: one channel, keys slot-permuted
-    static constexpr int SK = BN * DKP, SV = BN * DVP, SKT = 32 * MB * BNP;
-    static constexpr int STAGE = SK + SV + SKT;
+    static constexpr int SK = BN * ROWCH * 8, SV = BN * DVP;
+    static constexpr int STAGE = SK + SV;
     static constexpr int LDS_BYTES = 2 * STAGE * 2;
-    // loader: (4 keys x 8 channels) blocks of K and K_b (written row-major and transposed),
-    // 8-channel chunks of V
+    // loader: 8-channel chunks of K, K_b and V, one key row each
     static constexpr int CD = 2 * NKD, CR = 2 * NKR;
-    static constexpr int QUADS = BN / 4;
-    static constexpr int K_TASKS = QUADS * (CD + CR), V_TASKS = BN * CD;
+    static constexpr int K_TASKS = BN * (CD + CR), V_TASKS = BN * CD;
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
 #ifdef FB_Q1
@@ -57,16 +56,16 @@ struct DqCfg {
 
 template <class C>
 struct DqStage {
-    u32x4_t k[C::K_PT][4];
+    u32x4_t k[C::K_PT];
     u32x4_t v[C::V_PT];
 };
 
 template <class C>
 struct DqLoader {
-    // K task: quad of 4 keys x one 8-channel chunk of K (chunk < CD) or K_b
-    __device__ static __forceinline__ void ktask(int task, int &quad, int &ch, bool &is_b) {
-        quad = task % C::QUADS;
-        const int cc = task / C::QUADS;
+    // K task: one key row x one 8-channel chunk of K (chunk < CD) or K_b
+    __device__ static __forceinline__ void ktask(int task, int &row, int &ch, bool &is_b) {
+        row = task % C::BN;
+        const int cc = task / C::BN;
         is_b = cc >= C::CD;
         ch = is_b ? cc - C::CD : cc;
     }
@@ -76,18 +75,15 @@ struct DqLoader {
 #pragma unroll
         for (int i = 0; i < C::K_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
-            int quad, ch;
+            int row, ch;
             bool is_b;
-            ktask(task, quad, ch, is_b);
+            ktask(task, row, ch, is_b);
             const uint16_t *base = is_b ? kbbase : kbase;
             const int64_t ld = is_b ? a.kb.ss : a.k.ss;
             const int ncols = is_b ? a.r : a.d;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                st.k[i][j] = u32x4_t{0u, 0u, 0u, 0u};
-                if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS)
-                    st.k[i][j] = load_chunk<C::VEC>(base, ld, n0 + quad * 4 + j, a.Lk, ch * 8, ncols);
-            }
+            st.k[i] = u32x4_t{0u, 0u, 0u, 0u};
+            if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS)
+                st.k[i] = load_chunk<C::VEC>(base, ld, n0 + row, a.Lk, ch * 8, ncols);
         }
 #pragma unroll
         for (int i = 0; i < C::V_PT; ++i) {
@@ -100,28 +96,15 @@ struct DqLoader {
 
     __device__ static __forceinline__ void store(const DqStage<C> &st, uint16_t *stage, int tid,
                                                  const bool (&kok)[C::K_PT], const bool (&vok)[C::V_PT]) {
-        uint16_t *sK = stage, *sV = sK + C::SK, *sKt = sV + C::SV;
+        uint16_t *sK = stage, *sV = sK + C::SK;
 #pragma unroll
         for (int i = 0; i < C::K_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
-            int quad, ch;
+            int row, ch;
             bool is_b;
-            ktask(task, quad, ch, is_b);
-            if (kok[i]) {
-                const int col0 = (is_b ? 16 * C::NKD : 0) + ch * 8;
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    *reinterpret_cast<u32x4_t *>(sK + (quad * 4 + j) * C::DKP + col0) = st.k[i][j];
-                const int kcol = slot_of(quad * 4);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) { // channel col0 + e gets its four keys as one 8-byte store
-                    const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-                    u32x2_t pk;
-                    pk[0] = __builtin_amdgcn_perm(st.k[i][1][e >> 1], st.k[i][0][e >> 1], sel);
-                    pk[1] = __builtin_amdgcn_perm(st.k[i][3][e >> 1], st.k[i][2][e >> 1], sel);
-                    *reinterpret_cast<u32x2_t *>(sKt + (col0 + e) * C::BNP + kcol) = pk;
-                }
-            }
+            ktask(task, row, ch, is_b);
+            if (kok[i])
+                *reinterpret_cast<u32x4_t *>(sK + swz_off<C::ROWCH>(row, (is_b ? 2 * C::NKD : 0) + ch)) = st.k[i];
         }
 #pragma unroll
         for (int i = 0; i < C::V_PT; ++i) {
@@ -138,7 +121,6 @@ struct DqLoader {
 template <class C>
 struct DqFast {
     const uint16_t *kptr[C::K_PT], *vptr[C::V_PT];
-    uint32_t koff[C::K_PT][4];
     int64_t kinc[C::K_PT], vinc[C::V_PT];
     bool kok[C::K_PT], vok[C::V_PT];
 
@@ -147,16 +129,14 @@ struct DqFast {
 #pragma unroll
         for (int i = 0; i < C::K_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
-            int quad, ch;
+            int row, ch;
             bool is_b;
-            DqLoader<C>::ktask(task, quad, ch, is_b);
+            DqLoader<C>::ktask(task, row, ch, is_b);
             const uint16_t *base = is_b ? kbbase : kbase;
             const int64_t ld = is_b ? a.kb.ss : a.k.ss;
             kok[i] = task < C::K_TASKS && ch * 8 < (is_b ? a.r : a.d);
             kinc[i] = kok[i] ? ld * C::BN : 0;
-            kptr[i] = kok[i] ? base + (int64_t)n0 * ld + ch * 8 : kbase;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) koff[i][j] = kok[i] ? (uint32_t)((quad * 4 + j) * ld) : 0u;
+            kptr[i] = kok[i] ? base + (int64_t)(n0 + row) * ld + ch * 8 : kbase;
         }
 #pragma unroll
         for (int i = 0; i < C::V_PT; ++i) {
@@ -170,9 +150,7 @@ struct DqFast {
 
     __device__ __forceinline__ void load(DqStage<C> &st) const {
 #pragma unroll
-        for (int i = 0; i < C::K_PT; ++i)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) st.k[i][j] = *reinterpret_cast<const u32x4_t *>(kptr[i] + koff[i][j]);
+        for (int i = 0; i < C::K_PT; ++i) st.k[i] = *reinterpret_cast<const u32x4_t *>(kptr[i]);
 #pragma unroll
         for (int i = 0; i < C::V_PT; ++i) st.v[i] = *reinterpret_cast<const u32x4_t *>(vptr[i]);
     }
@@ -284,7 +262,7 @@ bwd_dq_kernel(const BwdArgs a) {
             fast.advance();
         }
 
-        const uint16_t *sK = stage0 + cur * C::STAGE, *sV = sK + C::SK, *sKt = sV + C::SV;
+        const uint16_t *sK = stage0 + cur * C::STAGE, *sV = sK + C::SK;
         const bool visible = !(a.causal && n0 > wq0 + 32 * C::QBLK - 1) && wq0 < a.Lq;
         if (visible) {
 #pragma unroll
@@ -292,7 +270,7 @@ bwd_dq_kernel(const BwdArgs a) {
                 u32x4_t ka[C::NK], va[C::NKD];
 #pragma unroll
                 for (int t = 0; t < C::NK; ++t)
-                    ka[t] = *reinterpret_cast<const u32x4_t *>(sK + (kb * 32 + c) * C::DKP + 16 * t + 8 * g);
+                    ka[t] = *reinterpret_cast<const u32x4_t *>(sK + swz_off<C::ROWCH>(kb * 32 + c, 2 * t + g));
 #pragma unroll
                 for (int t = 0; t < C::NKD; ++t)
                     va[t] = *reinterpret_cast<const u32x4_t *>(sV + (kb * 32 + c) * C::DVP + 16 * t + 8 * g);
@@ -340,8 +318,7 @@ bwd_dq_kernel(const BwdArgs a) {
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
                     for (int n = 0; n < C::MB; ++n) {
-                        const u32x4_t kt = *reinterpret_cast<const u32x4_t *>(sKt + (32 * n + c) * C::BNP + kb * 32 +
-                                                                             16 * t + 8 * g);
+                        const u32x4_t kt = lds_read_a_tr<C::ROWCH>(sK, kb * 32 + 16 * t, 32 * n, c, g);
 #pragma unroll
                         for (int qb = 0; qb < C::QBLK; ++qb) acc[qb][n] = T::mfma(kt, dsp[qb][t], acc[qb][n]);
                     }

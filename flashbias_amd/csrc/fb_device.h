@@ -128,6 +128,42 @@ __device__ __forceinline__ int slot_of(int x) {
     return (x & ~12) | ((x & 4) << 1) | ((x & 8) >> 1);
 }
 
+// LDS tiles that are read both row-wise (16-byte chunk of one row per lane: A operand with
+// rows = tile rows) and column-wise (ds_read_b64_tr_b16: A operand with rows = tile columns)
+// keep one row-major copy whose 16-byte chunks are XOR-swizzled by row, so that both access
+// patterns are free of bank conflicts.  ROWCH = chunks per row (8 -> 128-byte rows).
+__device__ __forceinline__ int swz_of(int row) { // 3-bit chunk swizzle from row bits 1, 2, 3
+    return ((row & 2) << 1) | ((row >> 2) & 1) | ((row >> 2) & 2);
+}
+template <int ROWCH>
+__device__ __forceinline__ int swz_off(int row, int chunk) { // element offset of a chunk
+    return (row * ROWCH + (chunk ^ swz_of(row))) * 8;
+}
+
+// Transposing LDS read.  Within each group of 16 lanes, lane 4a + b receives as element j the
+// b-th 16-bit element of the 8 bytes that lane 4j + a points at.  With lane 4j + a pointing at
+// tile[k0 + j][c0 + 4a ..], lane 4a + b gets tile[k0 .. k0 + 3][c0 + 4a + b]: four consecutive
+// rows of one column.
+__device__ __forceinline__ u32x2_t lds_read_tr4(const uint16_t *p) {
+    typedef short v4s_t __attribute__((ext_vector_type(4)));
+    const v4s_t r = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (v4s_t __attribute__((address_space(3))) *)(__attribute__((address_space(3))) const void *)p);
+    return __builtin_bit_cast(u32x2_t, r);
+}
+
+// A operand (rows = 32 tile columns starting at col0, contraction over 16 tile rows starting
+// at row0) for a B operand that comes straight from a C-layout register block: C-layout
+// element i of half-wave g is row 8 (i / 4) + 4 g + i % 4 of the 16, so each lane needs two
+// runs of four consecutive rows.
+template <int ROWCH>
+__device__ __forceinline__ u32x4_t lds_read_a_tr(const uint16_t *tile, int row0, int col0, int c, int g) {
+    const int chunk = (col0 >> 3) + 2 * (c >> 4) + ((c & 3) >> 1), within = 4 * (c & 1);
+    const int r = row0 + 4 * g + ((c & 15) >> 2);
+    const u32x2_t lo = lds_read_tr4(tile + swz_off<ROWCH>(r, chunk) + within);
+    const u32x2_t hi = lds_read_tr4(tile + swz_off<ROWCH>(r + 8, chunk) + within);
+    return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+}
+
 // Grid id -> logical work id such that the workgroups that land on one XCD (hardware hands
 // consecutive ids to the 8 XCDs round-robin) cover a contiguous range of logical ids and so
 // share K/V of the same (batch, head) in that XCD's L2.
