@@ -13,8 +13,8 @@
 //   P   = exp(S - lse)                                         (:670)
 //   dP  = dO V^T - delta      accumulator starts at -delta, read from LDS into place (:705-714)
 //   dS  = P * dP
-//   dV^T          += dO^T P              A = dO^T tile (LDS),      B = P registers   (:697)
-//   [dK | dK_b]^T += [Q | Q_b]^T dS      A = [Q | Q_b]^T tile (LDS), B = dS registers (:717-719)
+//   dV^T          += dO^T P              A = dO tile read column-wise (LDS),      B = P registers   (:697)
+//   [dK | dK_b]^T += [Q | Q_b]^T dS      A = [Q | Q_b] tile read column-wise (LDS), B = dS registers (:717-719)
 //
 // P and dS feed their MFMAs straight from the accumulator layout (no LDS round trip); every
 // A operand read from LDS is used for all KBW key blocks of the wave.  The accumulators are
@@ -33,16 +33,16 @@ struct DkvCfg {
     static constexpr int KBW = 1; // key blocks per wave
     static constexpr int BN = 32 * KBW * NWAVES;              // keys per workgroup
     static constexpr int QBLK = 2, BMQ = 32 * QBLK;           // queries per step
-    static constexpr int DKP = 16 * NK + 8;  // sQ row (elements)
-    static constexpr int DOP = 16 * NKD + 8; // sdO row
-    static constexpr int QTP = BMQ + 8;      // sQt / sdOt row (queries, slot-permuted)
-    static constexpr int SQ = BMQ * DKP, SDO = BMQ * DOP, SQT = 32 * MB * QTP, SDOT = 32 * NDV * QTP;
-    static constexpr int STAGE_ELEMS = SQ + SDO + SQT + SDOT + 4 * BMQ; // + lse2, -delta as fp32
+    // sQ row: [Q | Q_b] of one query, sdO row: dout of one query, both in swizzled 16-byte
+    // chunks; each tile is kept once and read row-wise (S, dP) and column-wise (dK, dV)
+    static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
+    static constexpr int ROWCHO = 2 * NKD <= 8 ? 8 : 16;
+    static constexpr int SQ = BMQ * ROWCH * 8, SDO = BMQ * ROWCHO * 8;
+    static constexpr int STAGE_ELEMS = SQ + SDO + 4 * BMQ; // + lse2, -delta as fp32
     static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2; // two stages
-    // loader tasks: (4 queries x 8 channels) blocks of Q, Q_b and dout
+    // loader tasks: 8-channel chunks of Q, Q_b and dout, one query row each
     static constexpr int CQ = 2 * NKD, CR = 2 * NKR, CO = 2 * NKD;
-    static constexpr int QUADS = BMQ / 4;
-    static constexpr int TASKS = QUADS * (CQ + CR + CO);
+    static constexpr int TASKS = BMQ * (CQ + CR + CO);
     static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
 #ifdef FB_W3
     static constexpr int WAVES_EU = 3;
@@ -53,15 +53,15 @@ struct DkvCfg {
 
 template <class C>
 struct DkvStage {
-    u32x4_t x[C::PT][4];
+    u32x4_t x[C::PT];
     float lse2, negd;
 };
 
-// task -> (kind, quad, chunk): kind 0 = Q, 1 = Q_b, 2 = dout
+// task -> (kind, row, chunk): kind 0 = Q, 1 = Q_b, 2 = dout
 template <class C>
 __device__ __forceinline__ void dkv_task(int task, int &kind, int &quad, int &ch) {
-    quad = task % C::QUADS;
-    const int cc = task / C::QUADS;
+    quad = task % C::BMQ;
+    const int cc = task / C::BMQ;
     if (cc < C::CQ) {
         kind = 0;
         ch = cc;
@@ -87,12 +87,9 @@ __device__ __forceinline__ void dkv_load_step(DkvStage<C> &st, const BwdArgs &a,
         const uint16_t *base = kind == 0 ? qbase : kind == 1 ? qbbase : dobase;
         const int64_t ld = kind == 0 ? a.q.ss : kind == 1 ? a.qb.ss : a.dout.ss;
         const int ncols = kind == 1 ? a.r : a.d;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            st.x[i][j] = u32x4_t{0u, 0u, 0u, 0u};
-            if (C::TASKS % C::NTHREADS == 0 || task < C::TASKS)
-                st.x[i][j] = load_chunk<C::VEC>(base, ld, m0 + quad * 4 + j, a.Lq, ch * 8, ncols);
-        }
+        st.x[i] = u32x4_t{0u, 0u, 0u, 0u};
+        if (C::TASKS % C::NTHREADS == 0 || task < C::TASKS)
+            st.x[i] = load_chunk<C::VEC>(base, ld, m0 + quad, a.Lq, ch * 8, ncols);
     }
     st.lse2 = INFINITY; // rows past the end: P = exp2(-inf) = 0
     st.negd = 0.f;
@@ -103,13 +100,12 @@ __device__ __forceinline__ void dkv_load_step(DkvStage<C> &st, const BwdArgs &a,
 }
 
 // Per-thread constants of the fast loader: a running global pointer per task (advanced by one
-// query step at a time) and the element offsets of the task's four rows.  Steps that lie
+// query step at a time).  Steps that lie
 // entirely inside the sequence are fetched with plain loads that nothing waits on until the
 // registers are written to LDS after the step's arithmetic.
 template <class C>
 struct DkvFast {
     const uint16_t *ptr[C::PT];
-    uint32_t off[C::PT][4];
     int64_t inc[C::PT];
     bool ok[C::PT];
 
@@ -125,18 +121,13 @@ struct DkvFast {
             const int ncols = kind == 1 ? a.r : a.d;
             ok[i] = task < C::TASKS && ch * 8 < ncols;
             inc[i] = ok[i] ? ld * C::BMQ : 0;
-            ptr[i] = ok[i] ? base + (int64_t)m0 * ld + ch * 8 : qbase;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) off[i][j] = ok[i] ? (uint32_t)((quad * 4 + j) * ld) : 0u;
+            ptr[i] = ok[i] ? base + (int64_t)(m0 + quad) * ld + ch * 8 : qbase;
         }
     }
 
     __device__ __forceinline__ void load(DkvStage<C> &st, const float *lse, const float *delta, int m0, int tid) {
 #pragma unroll
-        for (int i = 0; i < C::PT; ++i) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) st.x[i][j] = *reinterpret_cast<const u32x4_t *>(ptr[i] + off[i][j]);
-        }
+        for (int i = 0; i < C::PT; ++i) st.x[i] = *reinterpret_cast<const u32x4_t *>(ptr[i]);
         if (tid < C::BMQ) {
             st.lse2 = lse[m0 + tid];
             st.negd = delta[m0 + tid];
@@ -152,32 +143,18 @@ struct DkvFast {
 template <class C>
 __device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *stage, int tid, const bool (&ok)[C::PT],
                                                bool raw_stats) {
-    uint16_t *sQ = stage, *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
-    float *sStat = reinterpret_cast<float *>(sdOt + C::SDOT);
+    uint16_t *sQ = stage, *sdO = sQ + C::SQ;
+    float *sStat = reinterpret_cast<float *>(sdO + C::SDO);
 #pragma unroll
     for (int i = 0; i < C::PT; ++i) {
         const int task = tid + i * C::NTHREADS;
-        int kind, quad, ch;
-        dkv_task<C>(task, kind, quad, ch);
+        int kind, row, ch;
+        dkv_task<C>(task, kind, row, ch);
         if (ok[i]) { // chunks in the zero padding of the channel dim are never written (LDS cleared once)
-            // row-major copy (A operand of S and dP) ...
-            uint16_t *rm = kind == 2 ? sdO : sQ;
-            const int ld = kind == 2 ? C::DOP : C::DKP;
-            const int col0 = (kind == 1 ? 16 * C::NKD : 0) + ch * 8;
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                *reinterpret_cast<u32x4_t *>(rm + (quad * 4 + j) * ld + col0) = st.x[i][j];
-            // ... and transposed copy (A operand of dV^T and [dK|dK_b]^T), queries slot-permuted
-            uint16_t *tr = kind == 2 ? sdOt : sQt;
-            const int qcol = slot_of(quad * 4);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const uint32_t sel = (e & 1) ? 0x07060302u : 0x05040100u;
-                u32x2_t pk;
-                pk[0] = __builtin_amdgcn_perm(st.x[i][1][e >> 1], st.x[i][0][e >> 1], sel);
-                pk[1] = __builtin_amdgcn_perm(st.x[i][3][e >> 1], st.x[i][2][e >> 1], sel);
-                *reinterpret_cast<u32x2_t *>(tr + (col0 + e) * C::QTP + qcol) = pk;
-            }
+            if (kind == 2)
+                *reinterpret_cast<u32x4_t *>(sdO + swz_off<C::ROWCHO>(row, ch)) = st.x[i];
+            else
+                *reinterpret_cast<u32x4_t *>(sQ + swz_off<C::ROWCH>(row, (kind == 1 ? 2 * C::NKD : 0) + ch)) = st.x[i];
         }
     }
     if (tid < C::BMQ) { // the fast loader leaves lse and delta as read; convert here
@@ -287,8 +264,8 @@ bwd_dkv_kernel(const BwdArgs a) {
             fast.advance();
         }
         const uint16_t *sQ = stage0 + cur * C::STAGE_ELEMS;
-        const uint16_t *sdO = sQ + C::SQ, *sQt = sdO + C::SDO, *sdOt = sQt + C::SQT;
-        const float *sStat = reinterpret_cast<const float *>(sdOt + C::SDOT);
+        const uint16_t *sdO = sQ + C::SQ;
+        const float *sStat = reinterpret_cast<const float *>(sdO + C::SDO);
 
         const bool visible = !(a.causal && wk0 > m0 + C::BMQ - 1) && wk0 < a.Lk;
         if (visible) {
@@ -297,10 +274,10 @@ bwd_dkv_kernel(const BwdArgs a) {
                 u32x4_t qa[C::NK], da[C::NKD];
 #pragma unroll
                 for (int t = 0; t < C::NK; ++t)
-                    qa[t] = *reinterpret_cast<const u32x4_t *>(sQ + (qb * 32 + c) * C::DKP + 16 * t + 8 * g);
+                    qa[t] = *reinterpret_cast<const u32x4_t *>(sQ + swz_off<C::ROWCH>(qb * 32 + c, 2 * t + g));
 #pragma unroll
                 for (int t = 0; t < C::NKD; ++t)
-                    da[t] = *reinterpret_cast<const u32x4_t *>(sdO + (qb * 32 + c) * C::DOP + 16 * t + 8 * g);
+                    da[t] = *reinterpret_cast<const u32x4_t *>(sdO + swz_off<C::ROWCHO>(qb * 32 + c, 2 * t + g));
                 u32x4_t pp[C::KBW][2], pds[C::KBW][2]; // P and dS, packed, per 16-query step
 #pragma unroll
                 for (int kb = 0; kb < C::KBW; ++kb) {
@@ -356,15 +333,13 @@ bwd_dkv_kernel(const BwdArgs a) {
                 for (int t = 0; t < 2; ++t) {
 #pragma unroll
                     for (int n = 0; n < C::NDV; ++n) {
-                        const u32x4_t dot = *reinterpret_cast<const u32x4_t *>(sdOt + (32 * n + c) * C::QTP + qb * 32 +
-                                                                              16 * t + 8 * g);
+                        const u32x4_t dot = lds_read_a_tr<C::ROWCHO>(sdO, qb * 32 + 16 * t, 32 * n, c, g);
 #pragma unroll
                         for (int kb = 0; kb < C::KBW; ++kb) acc_dv[kb][n] = T::mfma(dot, pp[kb][t], acc_dv[kb][n]);
                     }
 #pragma unroll
                     for (int n = 0; n < C::MB; ++n) {
-                        const u32x4_t qt = *reinterpret_cast<const u32x4_t *>(sQt + (32 * n + c) * C::QTP + qb * 32 +
-                                                                             16 * t + 8 * g);
+                        const u32x4_t qt = lds_read_a_tr<C::ROWCH>(sQ, qb * 32 + 16 * t, 32 * n, c, g);
 #pragma unroll
                         for (int kb = 0; kb < C::KBW; ++kb) acc_dk[kb][n] = T::mfma(qt, pds[kb][t], acc_dk[kb][n]);
                     }
