@@ -1,4 +1,6 @@
-// delta = rowsum(o * dout), the memory-bound first step of the backward pass.
+// delta = rowsum(o * dout), the memory-bound first step of the backward pass.  The scratch
+// buffer receives what the two main kernels consume: -delta in its first B*H*Lq floats and
+// lse * log2(e) in the next B*H*Lq.
 // Replaces _bwd_preprocess_do_o_dot of the reference (flash_bias/flash_bias_triton.py:358-400).
 #include "fb_kernels.h"
 
@@ -32,7 +34,8 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a) {
                 acc += T::to_float((uint16_t)(x[e] >> 16)) * T::to_float((uint16_t)(y[e] >> 16));
             }
         }
-        a.delta[rix] = acc;
+        a.delta[rix] = -acc;
+        a.delta[rows + rix] = a.lse[rix] * kLog2e;
     }
 }
 

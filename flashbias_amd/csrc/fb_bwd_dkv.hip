@@ -5,13 +5,15 @@
 //
 // Key-stationary: one workgroup (4 waves) owns 64 * KBW consecutive keys of one
 // (batch, head), wave w owns KBW blocks of 32 of them, whose K, K_b and V stay in registers.
-// Queries are streamed in steps of 64 (two 32-blocks) through double-buffered LDS, the next
-// step prefetched into registers.  With lane = key, register = query (C layout of S with A = query rows from
+// Queries are streamed in steps of 64 (two 32-blocks) through a ring of three LDS stages that
+// global_load_lds fills directly, two steps ahead of the arithmetic (one step of arithmetic is
+// shorter than a trip to memory), without passing through registers.  With lane = key, register = query (C layout of S with A = query rows from
 // LDS, B = key registers):
 //
 //   S   = [Q | Q_b] [K | K_b]^T, the q k^T part times scale  (:638-641)
 //   P   = exp(S - lse)                                         (:670)
-//   dP  = dO V^T - delta      accumulator starts at -delta, read from LDS into place (:705-714)
+//   dP  = dO V^T - delta      accumulator starts at -delta, read from LDS into place (:705-714);
+//                             lse * log2(e) and -delta come from the preprocess step
 //   dS  = P * dP
 //   dV^T          += dO^T P              A = dO tile read column-wise (LDS),      B = P registers   (:697)
 //   [dK | dK_b]^T += [Q | Q_b]^T dS      A = [Q | Q_b] tile read column-wise (LDS), B = dS registers (:717-719)
@@ -38,29 +40,26 @@ struct DkvCfg {
     static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
     static constexpr int ROWCHO = 2 * NKD <= 8 ? 8 : 16;
     static constexpr int SQ = BMQ * ROWCH * 8, SDO = BMQ * ROWCHO * 8;
-    static constexpr int STAGE_ELEMS = SQ + SDO + 4 * BMQ; // + lse2, -delta as fp32
-    static constexpr int LDS_BYTES = 2 * STAGE_ELEMS * 2; // two stages
+    static constexpr int STAGE_ELEMS = SQ + SDO + 4 * BMQ; // + lse * log2(e), -delta as fp32
+    static constexpr int NSTAGE = 3;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_ELEMS * 2;
     // loader tasks: 8-channel chunks of Q, Q_b and dout, one query row each
     static constexpr int CQ = 2 * NKD, CR = 2 * NKR, CO = 2 * NKD;
     static constexpr int TASKS = BMQ * (CQ + CR + CO);
     static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
-#ifdef FB_W3
-    static constexpr int WAVES_EU = 3;
-#else
     static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 2 : 1;
-#endif
 };
 
 template <class C>
-struct DkvStage {
-    u32x4_t x[C::PT];
+struct DkvStage { // register staging of one step: only the element-wise loader uses x
+    u32x4_t x[C::VEC ? 1 : C::PT];
     float lse2, negd;
 };
 
 // task -> (kind, row, chunk): kind 0 = Q, 1 = Q_b, 2 = dout
 template <class C>
-__device__ __forceinline__ void dkv_task(int task, int &kind, int &quad, int &ch) {
-    quad = task % C::BMQ;
+__device__ __forceinline__ void dkv_task(int task, int &kind, int &row, int &ch) {
+    row = task % C::BMQ;
     const int cc = task / C::BMQ;
     if (cc < C::CQ) {
         kind = 0;
@@ -74,94 +73,154 @@ __device__ __forceinline__ void dkv_task(int task, int &kind, int &quad, int &ch
     }
 }
 
+// lse * log2(e) and -delta of query m0 + tid (as the preprocess step left them), for the first
+// BMQ threads; rows past the end get P = exp2(-inf) = 0.
+template <class C>
+__device__ __forceinline__ void dkv_load_stats(DkvStage<C> &st, const float *lse2, const float *negd, int m0, int Lq,
+                                               int tid) {
+    if (tid < C::BMQ) {
+        const bool ok = m0 + tid < Lq;
+        const int q = ok ? m0 + tid : Lq - 1;
+        const float l = lse2[q], d = negd[q];
+        st.lse2 = ok ? l : INFINITY;
+        st.negd = ok ? d : 0.f;
+    }
+}
+
+template <class C>
+__device__ __forceinline__ void dkv_store_stats(const DkvStage<C> &st, uint16_t *stage, int tid) {
+    float *sStat = reinterpret_cast<float *>(stage + C::SQ + C::SDO);
+    if (tid < C::BMQ) {
+        sStat[tid] = st.lse2;
+        sStat[C::BMQ + tid] = st.negd;
+    }
+}
+
+// Element-wise loader (tensors that are not 16-byte aligned, d or r not a multiple of 8):
+// clamped loads into registers, written to LDS after the step's arithmetic.
 template <class C>
 __device__ __forceinline__ void dkv_load_step(DkvStage<C> &st, const BwdArgs &a, const uint16_t *qbase,
-                                              const uint16_t *qbbase, const uint16_t *dobase, const float *lse,
-                                              const float *delta, int m0, int tid) {
+                                              const uint16_t *qbbase, const uint16_t *dobase, int m0, int tid) {
 #pragma unroll
-    for (int i = 0; i < C::PT; ++i) {
+    for (int i = 0; i < (C::VEC ? 1 : C::PT); ++i) {
         const int task = tid + i * C::NTHREADS;
-        int kind, quad, ch;
-        dkv_task<C>(task, kind, quad, ch);
+        int kind, row, ch;
+        dkv_task<C>(task, kind, row, ch);
         // one load per task: pick the tensor by lane (all three share the chunk geometry)
         const uint16_t *base = kind == 0 ? qbase : kind == 1 ? qbbase : dobase;
         const int64_t ld = kind == 0 ? a.q.ss : kind == 1 ? a.qb.ss : a.dout.ss;
         const int ncols = kind == 1 ? a.r : a.d;
         st.x[i] = u32x4_t{0u, 0u, 0u, 0u};
         if (C::TASKS % C::NTHREADS == 0 || task < C::TASKS)
-            st.x[i] = load_chunk<C::VEC>(base, ld, m0 + quad, a.Lq, ch * 8, ncols);
-    }
-    st.lse2 = INFINITY; // rows past the end: P = exp2(-inf) = 0
-    st.negd = 0.f;
-    if (tid < C::BMQ && m0 + tid < a.Lq) {
-        st.lse2 = lse[m0 + tid] * kLog2e;
-        st.negd = -delta[m0 + tid];
+            st.x[i] = load_chunk<false>(base, ld, m0 + row, a.Lq, ch * 8, ncols);
     }
 }
 
-// Per-thread constants of the fast loader: a running global pointer per task (advanced by one
-// query step at a time).  Steps that lie
-// entirely inside the sequence are fetched with plain loads that nothing waits on until the
-// registers are written to LDS after the step's arithmetic.
 template <class C>
-struct DkvFast {
-    const uint16_t *ptr[C::PT];
-    int64_t inc[C::PT];
-    bool ok[C::PT];
-
-    __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *qbase, const uint16_t *qbbase,
-                                         const uint16_t *dobase, int m0, int tid) {
-#pragma unroll
-        for (int i = 0; i < C::PT; ++i) {
-            const int task = tid + i * C::NTHREADS;
-            int kind, quad, ch;
-            dkv_task<C>(task, kind, quad, ch);
-            const uint16_t *base = kind == 0 ? qbase : kind == 1 ? qbbase : dobase;
-            const int64_t ld = kind == 0 ? a.q.ss : kind == 1 ? a.qb.ss : a.dout.ss;
-            const int ncols = kind == 1 ? a.r : a.d;
-            ok[i] = task < C::TASKS && ch * 8 < ncols;
-            inc[i] = ok[i] ? ld * C::BMQ : 0;
-            ptr[i] = ok[i] ? base + (int64_t)(m0 + quad) * ld + ch * 8 : qbase;
-        }
-    }
-
-    __device__ __forceinline__ void load(DkvStage<C> &st, const float *lse, const float *delta, int m0, int tid) {
-#pragma unroll
-        for (int i = 0; i < C::PT; ++i) st.x[i] = *reinterpret_cast<const u32x4_t *>(ptr[i]);
-        if (tid < C::BMQ) {
-            st.lse2 = lse[m0 + tid];
-            st.negd = delta[m0 + tid];
-        }
-    }
-
-    __device__ __forceinline__ void advance() {
-#pragma unroll
-        for (int i = 0; i < C::PT; ++i) ptr[i] += inc[i];
-    }
-};
-
-template <class C>
-__device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, uint16_t *stage, int tid, const bool (&ok)[C::PT],
-                                               bool raw_stats) {
+__device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, const BwdArgs &a, uint16_t *stage, int tid) {
     uint16_t *sQ = stage, *sdO = sQ + C::SQ;
-    float *sStat = reinterpret_cast<float *>(sdO + C::SDO);
 #pragma unroll
-    for (int i = 0; i < C::PT; ++i) {
+    for (int i = 0; i < (C::VEC ? 1 : C::PT); ++i) {
         const int task = tid + i * C::NTHREADS;
         int kind, row, ch;
         dkv_task<C>(task, kind, row, ch);
-        if (ok[i]) { // chunks in the zero padding of the channel dim are never written (LDS cleared once)
+        // chunks in the zero padding of the channel dim are never written (LDS cleared once)
+        if (task < C::TASKS && ch * 8 < (kind == 1 ? a.r : a.d)) {
             if (kind == 2)
                 *reinterpret_cast<u32x4_t *>(sdO + swz_off<C::ROWCHO>(row, ch)) = st.x[i];
             else
                 *reinterpret_cast<u32x4_t *>(sQ + swz_off<C::ROWCH>(row, (kind == 1 ? 2 * C::NKD : 0) + ch)) = st.x[i];
         }
     }
-    if (tid < C::BMQ) { // the fast loader leaves lse and delta as read; convert here
-        sStat[tid] = raw_stats ? st.lse2 * kLog2e : st.lse2;
-        sStat[C::BMQ + tid] = raw_stats ? -st.negd : st.negd;
-    }
 }
+
+// Direct loader (16-byte aligned tensors, d and r multiples of 8).  A global_load_lds of 16
+// bytes per lane writes lane i at LDS base + 16 i, so one instruction fills 64 consecutive
+// chunk positions of a tile and each lane fetches the global chunk that the swizzle puts at
+// its position.  Lanes whose position is channel padding stay switched off (those chunks keep
+// the zeros of the initial clear); rows past the end of the sequence re-read the last row,
+// which is harmless because their P is 0.  Each wave issues a quarter of the instructions.
+template <class C>
+struct DkvDirect {
+    static constexpr int NQI = C::BMQ * C::ROWCH / 64 / C::NWAVES;  // instructions per wave, [Q | Q_b] tile
+    static constexpr int NOI = C::BMQ * C::ROWCHO / 64 / C::NWAVES; // dout tile
+    static constexpr int N = NQI + NOI;
+    // waves 0 and 1 also fetch the step's lse * log2(e) and -delta rows (BMQ = 64 floats: one
+    // 4-byte copy per lane)
+    static constexpr int NS = 1;
+    const uint16_t *src[N]; // tensor base + channel offset of this lane's chunk
+    uint32_t ld[N];         // row stride of that tensor (elements)
+    int row[N];             // row of the step that this lane fetches
+    bool ok[N];
+    const float *stat;      // this wave's statistics row of the (batch, head), or null
+    int wave, lane;
+
+    __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *qbase, const uint16_t *qbbase,
+                                         const uint16_t *dobase, const float *lse2, const float *negd, int wave_,
+                                         int lane_) {
+        static_assert(C::BMQ == 64, "one statistics row per copy instruction");
+        wave = wave_;
+        lane = lane_;
+        stat = wave == 0 ? lse2 : wave == 1 ? negd : nullptr;
+#pragma unroll
+        for (int j = 0; j < NQI; ++j) {
+            const int p = (wave * NQI + j) * 64 + lane;
+            const int r = p / C::ROWCH, pos = p % C::ROWCH;
+            const int chunk = pos ^ swz_of(r);
+            const bool is_b = chunk >= 2 * C::NKD;
+            const int cc = is_b ? chunk - 2 * C::NKD : chunk;
+            row[j] = r;
+            ok[j] = is_b ? (cc < 2 * C::NKR && cc * 8 < a.r) : (cc * 8 < a.d);
+            src[j] = ok[j] ? (is_b ? qbbase : qbase) + cc * 8 : qbase;
+            ld[j] = ok[j] ? (uint32_t)(is_b ? a.qb.ss : a.q.ss) : 0u;
+        }
+#pragma unroll
+        for (int j = 0; j < NOI; ++j) {
+            const int p = (wave * NOI + j) * 64 + lane;
+            const int r = p / C::ROWCHO, pos = p % C::ROWCHO;
+            const int chunk = pos ^ swz_of(r);
+            row[NQI + j] = r;
+            ok[NQI + j] = chunk * 8 < a.d;
+            src[NQI + j] = ok[NQI + j] ? dobase + chunk * 8 : dobase;
+            ld[NQI + j] = ok[NQI + j] ? (uint32_t)a.dout.ss : 0u;
+        }
+    }
+
+    __device__ __forceinline__ void issue(uint16_t *stage, int m0, int Lq) const {
+        const uint32_t base = lds_addr_of(stage);
+#pragma unroll
+        for (int j = 0; j < N; ++j) {
+            const int q = min(m0 + row[j], Lq - 1);
+            const uint16_t *g = src[j] + (uint64_t)q * ld[j];
+            const uint32_t dst = base + 2 * (j < NQI ? (wave * NQI + j) * 512 : C::SQ + (wave * NOI + (j - NQI)) * 512);
+            if (ok[j]) lds_dma16(g, dst);
+        }
+        if (wave < 2) lds_dma4(stat + min(m0 + lane, Lq - 1), base + 2 * (C::SQ + C::SDO) + wave * (4 * C::BMQ));
+    }
+
+    // Loads of this wave that may stay in flight when the data of the step before them is needed.
+    template <bool KEEP>
+    __device__ __forceinline__ void wait_older() const {
+        if (!KEEP)
+            wait_vmcnt<0>();
+        else if (wave < 2)
+            wait_vmcnt<N + NS>();
+        else
+            wait_vmcnt<N>();
+    }
+
+    // A last step that runs past the sequence fetched clamped rows: give them P = 0.
+    __device__ __forceinline__ void fix_ragged(uint16_t *stage, int m0, int Lq, int tid) const {
+        if (m0 + C::BMQ > Lq) {
+            float *sStat = reinterpret_cast<float *>(stage + C::SQ + C::SDO);
+            if (tid < C::BMQ && m0 + tid >= Lq) {
+                sStat[tid] = INFINITY;
+                sStat[C::BMQ + tid] = 0.f;
+            }
+            barrier_lds();
+        }
+    }
+};
 
 template <class T>
 __device__ __forceinline__ float dkv_mask_at(const MaskDesc &m, const uint8_t *base, int query, int key, int Lq,
@@ -173,7 +232,7 @@ __device__ __forceinline__ float dkv_mask_at(const MaskDesc &m, const uint8_t *b
 }
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::WAVES_EU == 3 ? 0 : 1)))) void
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
 bwd_dkv_kernel(const BwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
@@ -199,8 +258,9 @@ bwd_dkv_kernel(const BwdArgs a) {
         qbbase = a.qb.ptr + b * a.qb.sb + h * a.qb.sh;
         kbbase = a.kb.ptr + b * a.kb.sb + h * a.kb.sh;
     }
-    const float *lse = a.lse + (int64_t)bh * a.Lq;
-    const float *delta = a.delta + (int64_t)bh * a.Lq;
+    // the preprocess step left -delta and lse * log2(e) in the scratch buffer
+    const float *negd = a.delta + (int64_t)bh * a.Lq;
+    const float *lse2 = a.delta + ((int64_t)a.B * a.H + bh) * a.Lq;
     const uint8_t *mbase = nullptr;
     if constexpr (C::MASK)
         mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
@@ -236,32 +296,48 @@ bwd_dkv_kernel(const BwdArgs a) {
     const int step0 = a.causal ? n0 / C::BMQ : 0;
     const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
 
-    {   // clear both stages once: the zero padding of the channel dimension is never rewritten
+    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
         u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
         for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
     }
     __syncthreads();
-    DkvFast<C> fast;
-    fast.init(a, qbase, qbbase, dobase, (step0 + 1) * C::BMQ, tid); // first prefetch is step0 + 1
+    // Step s is computed from stage (s - step0) % 3.  Direct loader: the tiles of step s + 2 are
+    // requested at the top of step s; element-wise loader: step s + 1 goes through registers.
+    constexpr int AHEAD = C::VEC ? 2 : 1;
+    DkvDirect<C> direct;
     DkvStage<C> st;
-    if (step0 < nsteps) {
-        dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, step0 * C::BMQ, tid);
-        dkv_store_step<C>(st, stage0, tid, fast.ok, false);
+    if constexpr (C::VEC) {
+        direct.init(a, qbase, qbbase, dobase, lse2, negd, wave, lane);
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k)
+            if (step0 + k < nsteps) direct.issue(stage0 + k * C::STAGE_ELEMS, (step0 + k) * C::BMQ, a.Lq);
+        // the first step's tiles must have landed; the second step's may still be in flight
+        if (step0 + 1 < nsteps)
+            direct.template wait_older<true>();
+        else
+            direct.template wait_older<false>();
+    } else if (step0 < nsteps) {
+        dkv_load_stats<C>(st, lse2, negd, step0 * C::BMQ, a.Lq, tid);
+        dkv_store_stats<C>(st, stage0, tid);
+        dkv_load_step<C>(st, a, qbase, qbbase, dobase, step0 * C::BMQ, tid);
+        dkv_store_step<C>(st, a, stage0, tid);
     }
     __syncthreads();
 
+    int cur = 0; // stage of the current step
     for (int step = step0; step < nsteps; ++step) {
         const int m0 = step * C::BMQ;
-        const int cur = (step - step0) & 1;
         const bool more = step + 1 < nsteps;
-        // next step: plain in-flight loads if it lies inside the sequence, clamped loads otherwise
-        const bool next_fast = C::VEC && m0 + 2 * C::BMQ <= a.Lq;
-        if (more) {
-            if (next_fast)
-                fast.load(st, lse, delta, m0 + C::BMQ, tid);
-            else
-                dkv_load_step<C>(st, a, qbase, qbbase, dobase, lse, delta, m0 + C::BMQ, tid);
-            fast.advance();
+        const int nxt = cur == C::NSTAGE - 1 ? 0 : cur + 1;
+        if constexpr (C::VEC) {
+            if (step + AHEAD < nsteps) {
+                const int tgt = nxt == C::NSTAGE - 1 ? 0 : nxt + 1; // the stage that step - 1 has left
+                direct.issue(stage0 + tgt * C::STAGE_ELEMS, m0 + AHEAD * C::BMQ, a.Lq);
+            }
+            direct.fix_ragged(stage0 + cur * C::STAGE_ELEMS, m0, a.Lq, tid);
+        } else if (more) {
+            dkv_load_stats<C>(st, lse2, negd, m0 + C::BMQ, a.Lq, tid);
+            dkv_load_step<C>(st, a, qbase, qbbase, dobase, m0 + C::BMQ, tid);
         }
         const uint16_t *sQ = stage0 + cur * C::STAGE_ELEMS;
         const uint16_t *sdO = sQ + C::SQ;
@@ -346,8 +422,21 @@ bwd_dkv_kernel(const BwdArgs a) {
                 }
             }
         }
-        if (more) dkv_store_step<C>(st, stage0 + (cur ^ 1) * C::STAGE_ELEMS, tid, fast.ok, next_fast);
-        __syncthreads();
+        if constexpr (C::VEC) {
+            // the next step's tiles must have landed; the one after may still be in flight
+            if (step + AHEAD < nsteps)
+                direct.template wait_older<true>();
+            else
+                direct.template wait_older<false>();
+            barrier_lds();
+        } else {
+            if (more) {
+                dkv_store_stats<C>(st, stage0 + nxt * C::STAGE_ELEMS, tid);
+                dkv_store_step<C>(st, a, stage0 + nxt * C::STAGE_ELEMS, tid);
+            }
+            __syncthreads();
+        }
+        cur = nxt;
     }
 
     // ---- epilogue: dv, dk (times scale), dk_bias for this lane's keys

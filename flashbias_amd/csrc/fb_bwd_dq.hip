@@ -226,8 +226,9 @@ bwd_dq_kernel(const BwdArgs a) {
         }
         const bool ok = query < a.Lq;
         const int64_t sidx = (int64_t)bh * a.Lq + (ok ? query : a.Lq - 1);
-        lse2[qb] = ok ? a.lse[sidx] * kLog2e : INFINITY; // rows past the end: P = exp2(-inf) = 0
-        negd[qb] = ok ? -a.delta[sidx] : 0.f;
+        // the preprocess step left -delta and lse * log2(e) in the scratch buffer
+        lse2[qb] = ok ? a.delta[(int64_t)a.B * a.H * a.Lq + sidx] : INFINITY; // rows past the end: P = exp2(-inf) = 0
+        negd[qb] = ok ? a.delta[sidx] : 0.f;
 #pragma unroll
         for (int n = 0; n < C::MB; ++n)
 #pragma unroll

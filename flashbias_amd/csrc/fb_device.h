@@ -164,6 +164,29 @@ __device__ __forceinline__ u32x4_t lds_read_a_tr(const uint16_t *tile, int row0,
     return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
 }
 
+// Direct global -> LDS copies (global_load_lds): lane i of the wave writes its 16 (or 4) bytes at
+// LDS byte address `lds` + 16 i (4 i); `lds` must be wave-uniform; switched-off lanes write
+// nothing.  They are issued through inline assembly so that the compiler's wait-count pass does
+// not know them: it would make every later LDS read wait for all of them, and the point is to
+// keep them in flight for more than one step.  The price: they count in vmcnt like any load, in
+// issue order, and the kernel must wait for them itself (wait_vmcnt) before the barrier that
+// publishes the data.
+__device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
+    return (uint32_t)(size_t)(__attribute__((address_space(3))) const void *)p;
+}
+__device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(g) : "memory");
+}
+__device__ __forceinline__ void lds_dma4(const void *g, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds), "v"(g) : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() { // at most N vector memory loads of this wave still in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+// Workgroup barrier that only waits for this wave's LDS operations (not for loads in flight).
+__device__ __forceinline__ void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Grid id -> logical work id such that the workgroups that land on one XCD (hardware hands
 // consecutive ids to the 8 XCDs round-robin) cover a contiguous range of logical ids and so
 // share K/V of the same (batch, head) in that XCD's L2.

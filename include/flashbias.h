@@ -78,7 +78,7 @@ typedef struct fb_params {
     fb_tensor dq, dk, dv;       /* bwd out */
     fb_tensor dq_bias, dk_bias; /* bwd out, full (B, L, H, r) shape: the caller reduces over
                                    broadcast dims */
-    float *delta;               /* (B, H, Lq) fp32 scratch, written by the backward */
+    float *delta;               /* (2, B, H, Lq) fp32 scratch, written by the backward: -delta, lse * log2(e) */
 } fb_params;
 
 /* Library / ABI version. */
@@ -104,7 +104,8 @@ int fb_fwd(const fb_params *p, void *stream);
 int fb_bwd(const fb_params *p, void *stream);
 
 /* The phases of fb_bwd, exported so that a harness can time them separately.
- *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400)
+ *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400); fills the
+ *                      scratch with -delta (first B*H*Lq floats) and lse * log2(e) (next B*H*Lq)
  *   fb_bwd_dkv:        recompute P from lse; dk, dv, dk_bias, one workgroup per key tile
  *                      (_bwd_kernel / _bwd_kernel_one_col_block, :450-1097, minus dq)
  *   fb_bwd_dq:         recompute P from lse; dq, dq_bias, one workgroup per query tile
