@@ -134,25 +134,17 @@ __device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, const BwdA
     }
 }
 
-// Direct loader (16-byte aligned tensors, d and r multiples of 8).  A global_load_lds of 16
-// bytes per lane writes lane i at LDS base + 16 i, so one instruction fills 64 consecutive
-// chunk positions of a tile and each lane fetches the global chunk that the swizzle puts at
-// its position.  Lanes whose position is channel padding stay switched off (those chunks keep
-// the zeros of the initial clear); rows past the end of the sequence re-read the last row,
-// which is harmless because their P is 0.  Each wave issues a quarter of the instructions.
+// Direct loader (16-byte aligned tensors, d and r multiples of 8): the [Q | Q_b] and dout
+// tiles of a step plus its statistics rows, copied straight into an LDS stage.
 template <class C>
 struct DkvDirect {
-    static constexpr int NQI = C::BMQ * C::ROWCH / 64 / C::NWAVES;  // instructions per wave, [Q | Q_b] tile
-    static constexpr int NOI = C::BMQ * C::ROWCHO / 64 / C::NWAVES; // dout tile
-    static constexpr int N = NQI + NOI;
+    TileDma<C::BMQ, C::ROWCH, C::NWAVES> q;
+    TileDma<C::BMQ, C::ROWCHO, C::NWAVES> d;
+    static constexpr int N = decltype(q)::NI + decltype(d)::NI;
     // waves 0 and 1 also fetch the step's lse * log2(e) and -delta rows (BMQ = 64 floats: one
     // 4-byte copy per lane)
     static constexpr int NS = 1;
-    const uint16_t *src[N]; // tensor base + channel offset of this lane's chunk
-    uint32_t ld[N];         // row stride of that tensor (elements)
-    int row[N];             // row of the step that this lane fetches
-    bool ok[N];
-    const float *stat;      // this wave's statistics row of the (batch, head), or null
+    const float *stat; // this wave's statistics row of the (batch, head), or null
     int wave, lane;
 
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *qbase, const uint16_t *qbbase,
@@ -162,39 +154,14 @@ struct DkvDirect {
         wave = wave_;
         lane = lane_;
         stat = wave == 0 ? lse2 : wave == 1 ? negd : nullptr;
-#pragma unroll
-        for (int j = 0; j < NQI; ++j) {
-            const int p = (wave * NQI + j) * 64 + lane;
-            const int r = p / C::ROWCH, pos = p % C::ROWCH;
-            const int chunk = pos ^ swz_of(r);
-            const bool is_b = chunk >= 2 * C::NKD;
-            const int cc = is_b ? chunk - 2 * C::NKD : chunk;
-            row[j] = r;
-            ok[j] = is_b ? (cc < 2 * C::NKR && cc * 8 < a.r) : (cc * 8 < a.d);
-            src[j] = ok[j] ? (is_b ? qbbase : qbase) + cc * 8 : qbase;
-            ld[j] = ok[j] ? (uint32_t)(is_b ? a.qb.ss : a.q.ss) : 0u;
-        }
-#pragma unroll
-        for (int j = 0; j < NOI; ++j) {
-            const int p = (wave * NOI + j) * 64 + lane;
-            const int r = p / C::ROWCHO, pos = p % C::ROWCHO;
-            const int chunk = pos ^ swz_of(r);
-            row[NQI + j] = r;
-            ok[NQI + j] = chunk * 8 < a.d;
-            src[NQI + j] = ok[NQI + j] ? dobase + chunk * 8 : dobase;
-            ld[NQI + j] = ok[NQI + j] ? (uint32_t)a.dout.ss : 0u;
-        }
+        q.init(qbase, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? qbbase : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane);
+        d.init(dobase, a.dout.ss, a.d, C::ROWCHO, nullptr, 0, 0, wave, lane);
     }
 
     __device__ __forceinline__ void issue(uint16_t *stage, int m0, int Lq) const {
         const uint32_t base = lds_addr_of(stage);
-#pragma unroll
-        for (int j = 0; j < N; ++j) {
-            const int q = min(m0 + row[j], Lq - 1);
-            const uint16_t *g = src[j] + (uint64_t)q * ld[j];
-            const uint32_t dst = base + 2 * (j < NQI ? (wave * NQI + j) * 512 : C::SQ + (wave * NOI + (j - NQI)) * 512);
-            if (ok[j]) lds_dma16(g, dst);
-        }
+        q.issue(base, m0, Lq);
+        d.issue(base + 2 * C::SQ, m0, Lq);
         if (wave < 2) lds_dma4(stat + min(m0 + lane, Lq - 1), base + 2 * (C::SQ + C::SDO) + wave * (4 * C::BMQ));
     }
 
@@ -378,6 +345,8 @@ bwd_dkv_kernel(const BwdArgs a) {
                     for (int t = 0; t < C::NKD; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(da[t], vreg[kb][t], dp);
+                    // the softmax scale multiplies the fp32 q k^T accumulator before the bias steps
+                    // (one chain keeps this kernel at three waves per SIMD)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[v] *= a.scale;
 #pragma unroll

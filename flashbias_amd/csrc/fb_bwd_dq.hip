@@ -15,8 +15,8 @@
 //
 // so dS^T goes from the accumulator layout straight into the next MFMA and [dQ | dQ_b]^T stays
 // in registers for the whole key loop: each output element is written exactly once, in a fixed
-// summation order (bit-reproducible).  scale * q is split into hi + lo 16-bit parts as in the
-// forward; dq is multiplied by the scale in the epilogue, dq_bias is not (:728-732).
+// summation order (bit-reproducible).  The softmax scale multiplies the fp32 q k^T accumulator as
+// in the forward; dq is multiplied by the scale in the epilogue, dq_bias is not (:728-732).
 #include "fb_kernels.h"
 
 namespace fb {
@@ -206,7 +206,7 @@ bwd_dq_kernel(const BwdArgs a) {
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
     // ---- query-side operands, resident in registers
-    u32x4_t qhi[C::QBLK][C::NKD], qlo[C::QBLK][C::NKD], qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
+    u32x4_t qr[C::QBLK][C::NKD], qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
     u32x4_t dor[C::QBLK][C::NKD];
     float negd[C::QBLK], lse2[C::QBLK]; // -delta and lse * log2(e) of this lane's queries
     f32x16_t acc[C::QBLK][C::MB];
@@ -215,8 +215,7 @@ bwd_dq_kernel(const BwdArgs a) {
         const int query = wq0 + qb * 32 + c;
 #pragma unroll
         for (int t = 0; t < C::NKD; ++t) {
-            split_scaled<T>(load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d), a.scale, qhi[qb][t],
-                            qlo[qb][t]);
+            qr[qb][t] = load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d);
             dor[qb][t] = load_chunk<C::VEC>(dobase, a.dout.ss, query, a.Lq, 16 * t + 8 * g, a.d);
         }
         if constexpr (C::NKR > 0) {
@@ -281,14 +280,21 @@ bwd_dq_kernel(const BwdArgs a) {
                     f32x16_t s, dp;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
+                    // q k^T and q_b k_b^T: two independent MFMA chains, joined by one FMA per score
+                    // that applies the softmax scale in fp32 (:638-641)
 #pragma unroll
-                    for (int t = 0; t < C::NK; ++t) {
-                        if (t < C::NKD) {
-                            s = T::mfma(ka[t], qhi[qb][t], s);
-                            s = T::mfma(ka[t], qlo[qb][t], s);
-                        } else {
-                            s = T::mfma(ka[t], qbr[qb][t - C::NKD], s);
-                        }
+                    for (int t = 0; t < C::NKD; ++t) s = T::mfma(ka[t], qr[qb][t], s);
+                    if constexpr (C::NKR > 0) {
+                        f32x16_t sb;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) sb[v] = 0.f;
+#pragma unroll
+                        for (int t = C::NKD; t < C::NK; ++t) sb = T::mfma(ka[t], qbr[qb][t - C::NKD], sb);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) s[v] = __builtin_fmaf(s[v], a.scale, sb[v]);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) s[v] *= a.scale;
                     }
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], dp);

@@ -187,6 +187,51 @@ __device__ __forceinline__ void wait_vmcnt() { // at most N vector memory loads 
 // Workgroup barrier that only waits for this wave's LDS operations (not for loads in flight).
 __device__ __forceinline__ void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// One wave's share of the direct copies that fill a swizzled LDS tile of ROWS rows x ROWCH
+// 16-byte chunks from one or two row-major tensors: chunks [0, split) of a tile row come from
+// tensor A (channels 8 * chunk ..), chunks from `split` on from tensor B.  One copy
+// instruction fills 64 consecutive chunk positions of the tile and each lane fetches the global
+// chunk that the swizzle puts at its position.  Lanes whose position is channel padding stay
+// switched off (those chunks keep the zeros of the initial clear); rows past the end of the
+// tensor re-read its last row.  The NWAVES waves of the workgroup issue equal shares.
+template <int ROWS, int ROWCH, int NWAVES>
+struct TileDma {
+    static constexpr int NI = ROWS * ROWCH / 64 / NWAVES; // copy instructions per wave
+    static_assert(NI * 64 * NWAVES == ROWS * ROWCH, "tile must split evenly over the waves");
+    const uint16_t *src[NI]; // tensor base + channel offset of this lane's chunk
+    uint32_t ld[NI];         // row stride of that tensor (elements)
+    int row[NI];             // tile row this lane fetches
+    bool ok[NI];
+    int wave;
+
+    __device__ __forceinline__ void init(const uint16_t *a, int64_t lda, int ncols_a, int split, const uint16_t *b,
+                                         int64_t ldb, int ncols_b, int wave_, int lane) {
+        wave = wave_;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int p = (wave * NI + j) * 64 + lane;
+            const int r = p / ROWCH, pos = p % ROWCH;
+            const int chunk = pos ^ swz_of(r);
+            const bool is_b = chunk >= split;
+            const int cc = is_b ? chunk - split : chunk;
+            row[j] = r;
+            ok[j] = is_b ? (b != nullptr && cc * 8 < ncols_b) : (cc * 8 < ncols_a);
+            src[j] = ok[j] ? (is_b ? b : a) + cc * 8 : a;
+            ld[j] = ok[j] ? (uint32_t)(is_b ? ldb : lda) : 0u;
+        }
+    }
+
+    // tile <- tensor rows [r0, r0 + ROWS), clamped to nrows - 1
+    __device__ __forceinline__ void issue(uint32_t lds_tile, int r0, int nrows) const {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+            const int q = min(r0 + row[j], nrows - 1);
+            const uint16_t *g = src[j] + (uint64_t)q * ld[j];
+            if (ok[j]) lds_dma16(g, lds_tile + (wave * NI + j) * 1024);
+        }
+    }
+};
+
 // Grid id -> logical work id such that the workgroups that land on one XCD (hardware hands
 // consecutive ids to the 8 XCDs round-robin) cover a contiguous range of logical ids and so
 // share K/V of the same (batch, head) in that XCD's L2.

@@ -16,16 +16,14 @@
 // zero-padded to 16-wide MFMA steps.
 //
 // Softmax scale: the reference multiplies the fp32 q k^T accumulator by the scale and never
-// scales the bias product (flash_bias_triton.py:246-256).  Here scale * q is formed in fp32 when
-// the query operand is loaded and split into two 16-bit parts hi + lo (hi = round(x),
-// lo = round(x - hi)), both contracted against the same key registers: the product carries 16
-// mantissa bits of scale * q, the bias factors stay untouched, and the inner loop needs no
-// multiply per score.
+// scales the bias product (flash_bias_triton.py:246-256).  Same here: q k^T and q_b k_b^T are two
+// separate (and therefore independent, shorter) MFMA chains, joined by one fp32 FMA per score.
+// Measured on MI355X this beats folding the scale into the query operand (which needs a second,
+// low-order MFMA per step): the matrix pipe is the scarcer resource when two waves share a SIMD.
 //
-// The VALU, not the MFMA pipe, bounds this kernel at d = 32, so the per-score work is kept to:
-// max3, fma + exp2, convert, and a 2-way dot for the row sum; the running reference of the
-// softmax only moves when a row maximum grows by more than 2^8 (then p <= 256, exact enough in
-// fp32 / 16-bit), so the accumulator rescale is rare.
+// Per score the VALU does: fma (scale), max3, fma + exp2, convert, add (row sum); the running
+// reference of the softmax only moves when a row maximum grows by more than 2^8 (then
+// p <= 256, exact enough in fp32 / 16-bit), so the accumulator rescale is rare.
 #include "fb_kernels.h"
 
 namespace fb {
@@ -248,7 +246,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
     // ---- query operands, resident in registers for the whole key loop
-    u32x4_t qhi[C::QB][C::NKD], qlo[C::QB][C::NKD], qbr[C::QB][C::NKR > 0 ? C::NKR : 1];
+    u32x4_t qr[C::QB][C::NKD], qbr[C::QB][C::NKR > 0 ? C::NKR : 1];
     f32x16_t acc_o[C::QB][C::NDV];
     float m_ref[C::QB]; // reference of the exponentials (natural units), lags the true row max
     float m2[C::QB];    // m_ref * log2(e), 0 while the row has seen no finite score
@@ -258,8 +256,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         const int query = wq0 + 32 * qb + c;
 #pragma unroll
         for (int t = 0; t < C::NKD; ++t)
-            split_scaled<T>(load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d), a.scale, qhi[qb][t],
-                            qlo[qb][t]);
+            qr[qb][t] = load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d);
         if constexpr (C::NKR > 0) {
 #pragma unroll
             for (int t = 0; t < C::NKR; ++t)
@@ -342,21 +339,24 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                 f32x16_t s[C::KBLK];
 #pragma unroll
                 for (int kb = 0; kb < C::KBLK; ++kb) {
-                    f32x16_t acc;
+                    // the q k^T part and the bias part are two independent MFMA chains, joined by
+                    // one FMA per score that applies the softmax scale in fp32 (:246-256)
+                    f32x16_t acc, accb;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+                    for (int v = 0; v < 16; ++v) acc[v] = accb[v] = 0.f;
 #pragma unroll
                     for (int t = 0; t < C::NK; ++t) {
                         const u32x4_t kf = t < C::KPRE ? ka[kb][t < C::KPRE ? t : 0]
                                                        : *reinterpret_cast<const u32x4_t *>(
                                                              sK + (sub * C::BSUB + kb * 32 + c) * C::DKP + 16 * t + 8 * g);
-                        if (t < C::NKD) {
-                            acc = T::mfma(kf, qhi[qb][t], acc);
-                            acc = T::mfma(kf, qlo[qb][t], acc);
-                        } else {
-                            acc = T::mfma(kf, qbr[qb][t - C::NKD], acc);
-                        }
+                        if (t < C::NKD)
+                            acc = T::mfma(kf, qr[qb][t], acc);
+                        else
+                            accb = T::mfma(kf, qbr[qb][t - C::NKD], accb);
                     }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        acc[v] = C::NKR > 0 ? __builtin_fmaf(acc[v], a.scale, accb[v]) : acc[v] * a.scale;
                     s[kb] = acc;
                 }
                 // ---- additive mask, then -inf for keys past the end and causal-hidden pairs
