@@ -34,12 +34,23 @@ def _to_dev(w, dev):
     return {n: (t.to(dev) if isinstance(t, torch.Tensor) else t) for n, t in w.items()}
 
 
-def _time_events(fn, steps, warmup):
-    """Average milliseconds of fn() measured with events on the current stream."""
+def _time_events(fn, steps, warmup, isolated=False):
+    """Average milliseconds of fn() measured with events on the current stream.  isolated: one
+    event pair per call, so that the tail of one launch cannot overlap the head of the next (what
+    a kernel trace reports as a launch's duration); otherwise one pair around all the calls
+    (throughput of back-to-back launches)."""
     import torch
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    if isolated:
+        pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for start, end in pairs:
+            start.record()
+            fn()
+            end.record()
+        torch.cuda.synchronize()
+        return sum(start.elapsed_time(end) for start, end in pairs) / steps
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(steps):
@@ -125,7 +136,7 @@ def headline(args):
 
     f_fwd, f_bwd = workloads.flops(hl["B"], hl["H"], hl["L"], hl["L"], hl["d"], hl["r"])
     phases, keep = _phase_timers({n: (t.detach() if isinstance(t, torch.Tensor) else t) for n, t in w.items()}, dev)
-    ms = {name: _time_events(fn, args.steps, max(1, args.warmup)) for name, fn in phases.items()}
+    ms = {name: _time_events(fn, args.steps, max(1, args.warmup), isolated=True) for name, fn in phases.items()}
     # dominant kernel: dk/dv/dk_bias.  Its algorithmic share of the backward: S recompute
     # (d + r), dP (d), dV (d), dK|dK_b (d + r) of the 2 B H L^2 (5d + 3r); the dq kernel carries
     # the dQ|dQ_b product (d + r) and, beyond the algorithmic count, a second S / dP recompute.
