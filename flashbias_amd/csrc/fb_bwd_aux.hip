@@ -39,15 +39,73 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a) {
     }
 }
 
-hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream) {
+// Coalesced variant for 16-byte aligned tensors whose rows are 1, 2, 4, 8 or 16 chunks of 8
+// channels: one thread per chunk (consecutive threads read consecutive 16 bytes of a row), the
+// CH partial sums of a row are added across neighbouring lanes.
+template <class T, int CH>
+__global__ __launch_bounds__(256) void bwd_preprocess_chunks_kernel(const BwdArgs a) {
     const int64_t rows = (int64_t)a.B * a.H * a.Lq;
+    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t cix = gid; cix < rows * CH; cix += nthreads) { // rows * CH is a multiple of CH: whole rows per pass
+        const int c = (int)(cix % CH);
+        const int64_t r = cix / CH; // rows in memory order (b, i, h): neighbouring heads are adjacent
+        const int h = (int)(r % a.H);
+        const int i = (int)((r / a.H) % a.Lq);
+        const int b = (int)(r / ((int64_t)a.H * a.Lq));
+        const uint16_t *orow = a.o.ptr + b * a.o.sb + h * a.o.sh + (int64_t)i * a.o.ss;
+        const uint16_t *drow = a.dout.ptr + b * a.dout.sb + h * a.dout.sh + (int64_t)i * a.dout.ss;
+        float acc = 0.f;
+        if (c * 8 < a.d) {
+            const u32x4_t x = *reinterpret_cast<const u32x4_t *>(orow + c * 8);
+            const u32x4_t y = *reinterpret_cast<const u32x4_t *>(drow + c * 8);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc += T::to_float((uint16_t)(x[e] & 0xffffu)) * T::to_float((uint16_t)(y[e] & 0xffffu));
+                acc += T::to_float((uint16_t)(x[e] >> 16)) * T::to_float((uint16_t)(y[e] >> 16));
+            }
+        }
+#pragma unroll
+        for (int m = 1; m < CH; m <<= 1) acc += __shfl_xor(acc, m, 64);
+        if (c == 0) {
+            const int64_t rix = ((int64_t)b * a.H + h) * a.Lq + i;
+            a.delta[rix] = -acc;
+            a.delta[rows + rix] = a.lse[rix] * kLog2e;
+        }
+    }
+}
+
+template <class T>
+static void launch_preprocess_t(const BwdArgs &a, hipStream_t stream) {
+    const int64_t rows = (int64_t)a.B * a.H * a.Lq;
+    const bool vec = a.o.vec_ok && a.dout.vec_ok && a.d % 8 == 0;
+    const int chunks = (a.d + 7) / 8;
+    int ch = 1;
+    while (ch < chunks) ch <<= 1;
+    if (vec && ch <= 16) {
+        int64_t blocks = (rows * ch + 255) / 256;
+        if (blocks > 262144) blocks = 262144; // grid-stride beyond that; 256 * blocks stays a multiple of ch
+        const dim3 grid((unsigned)blocks), block(256);
+        switch (ch) {
+        case 1: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 1>), grid, block, 0, stream, a); break;
+        case 2: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 2>), grid, block, 0, stream, a); break;
+        case 4: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 4>), grid, block, 0, stream, a); break;
+        case 8: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 8>), grid, block, 0, stream, a); break;
+        default: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 16>), grid, block, 0, stream, a); break;
+        }
+        return;
+    }
     int64_t blocks = (rows + 255) / 256;
     if (blocks > 65536) blocks = 65536;
     if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(bwd_preprocess_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+}
+
+hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream) {
     if (bf16)
-        hipLaunchKernelGGL(bwd_preprocess_kernel<BF16>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        launch_preprocess_t<BF16>(a, stream);
     else
-        hipLaunchKernelGGL(bwd_preprocess_kernel<F16>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        launch_preprocess_t<F16>(a, stream);
     return hipGetLastError();
 }
 
