@@ -77,6 +77,9 @@ fb::MaskDesc dev_mask(const fb_params *p) {
     m.sm = p->mask_type == FB_MASK_MATRIX ? p->mask.stride_s : 0;
     m.type = p->mask_type;
     m.is_f32 = p->mask_dtype == FB_F32;
+    const uintptr_t align = m.is_f32 ? 16 : 8; // four consecutive keys
+    m.vec_ok = p->mask_type && reinterpret_cast<uintptr_t>(m.ptr) % align == 0 && m.sb % 4 == 0 && m.sh % 4 == 0 &&
+               m.sm % 4 == 0;
     return m;
 }
 

@@ -189,15 +189,6 @@ struct DkvDirect {
     }
 };
 
-template <class T>
-__device__ __forceinline__ float dkv_mask_at(const MaskDesc &m, const uint8_t *base, int query, int key, int Lq,
-                                             int Lk) {
-    if (key >= Lk || query >= Lq) return 0.f;
-    const int64_t off = (m.type == 2 ? (int64_t)query * m.sm : 0) + key;
-    if (m.is_f32) return reinterpret_cast<const float *>(base)[off];
-    return T::to_float(reinterpret_cast<const uint16_t *>(base)[off]);
-}
-
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
 bwd_dkv_kernel(const BwdArgs a) {
@@ -339,6 +330,9 @@ bwd_dkv_kernel(const BwdArgs a) {
                             dp[4 * bq + e] = d4[e];
                         }
                     }
+                    // additive mask: requested before the MFMAs, added by the FMA that applies the scale
+                    f32x16_t mk;
+                    if constexpr (C::MASK) mask_block_queries<T>(a.mask, mbase, m0 + qb * 32, g, key, a.Lq, a.Lk, mk);
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[v] = 0.f;
 #pragma unroll
@@ -348,15 +342,9 @@ bwd_dkv_kernel(const BwdArgs a) {
                     // the softmax scale multiplies the fp32 q k^T accumulator before the bias steps
                     // (one chain keeps this kernel at three waves per SIMD)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] *= a.scale;
+                    for (int v = 0; v < 16; ++v) s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mk[v]) : s[v] * a.scale;
 #pragma unroll
                     for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
-                    if constexpr (C::MASK) {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v)
-                            s[v] += dkv_mask_at<T>(a.mask, mbase, m0 + qb * 32 + 8 * (v >> 2) + 4 * g + (v & 3), key,
-                                                   a.Lq, a.Lk);
-                    }
                     const bool edge = (wk0 + kb * 32 + 32 > a.Lk) || (a.causal && wk0 + kb * 32 + 31 > m0 + qb * 32);
                     if (edge) {
 #pragma unroll
@@ -486,8 +474,11 @@ static hipError_t launch_dkv_vec(const BwdArgs &a0, hipStream_t stream) {
 
 template <class T, int NKD, int NKR, int NDV>
 static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
+    // the direct loader keeps row strides in 32 bits
+    const int64_t lim = (int64_t)1 << 31;
     const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
-                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0)) && a.q.ss < lim && a.dout.ss < lim &&
+                     (a.r == 0 || a.qb.ss < lim);
     if (a.mask.type)
         return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_dkv_vec<T, NKD, NKR, NDV, false, true>(a, stream);

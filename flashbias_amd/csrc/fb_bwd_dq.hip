@@ -163,15 +163,6 @@ struct DqFast {
     }
 };
 
-template <class T>
-__device__ __forceinline__ float dq_mask_at(const MaskDesc &m, const uint8_t *base, int query, int key, int Lq,
-                                            int Lk) {
-    if (key >= Lk || query >= Lq) return 0.f;
-    const int64_t off = (m.type == 2 ? (int64_t)query * m.sm : 0) + key;
-    if (m.is_f32) return reinterpret_cast<const float *>(base)[off];
-    return T::to_float(reinterpret_cast<const uint16_t *>(base)[off]);
-}
-
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU))) void
 bwd_dq_kernel(const BwdArgs a) {
@@ -278,33 +269,37 @@ bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
                 for (int qb = 0; qb < C::QBLK; ++qb) {
                     f32x16_t s, dp;
+                    const int query = wq0 + qb * 32 + c;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
                     // q k^T and q_b k_b^T: two independent MFMA chains, joined by one FMA per score
-                    // that applies the softmax scale in fp32 (:638-641)
-#pragma unroll
-                    for (int t = 0; t < C::NKD; ++t) s = T::mfma(ka[t], qr[qb][t], s);
-                    if constexpr (C::NKR > 0) {
+                    // that applies the softmax scale in fp32 (:638-641); an additive mask is the
+                    // initial value of the bias chain
+                    if constexpr (C::NKR > 0 || C::MASK) {
                         f32x16_t sb;
+                        if constexpr (C::MASK) {
+                            const uint8_t *mrow =
+                                mbase + (a.mask.type == 2 ? (int64_t)min(query, a.Lq - 1) * a.mask.sm : 0) *
+                                            (a.mask.is_f32 ? 4 : 2);
+                            mask_block_keys<T>(a.mask, mrow, n0 + kb * 32, g, a.Lk, sb);
+                        } else {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) sb[v] = 0.f;
+                            for (int v = 0; v < 16; ++v) sb[v] = 0.f;
+                        }
+#pragma unroll
+                        for (int t = 0; t < C::NKD; ++t) s = T::mfma(ka[t], qr[qb][t], s);
 #pragma unroll
                         for (int t = C::NKD; t < C::NK; ++t) sb = T::mfma(ka[t], qbr[qb][t - C::NKD], sb);
 #pragma unroll
                         for (int v = 0; v < 16; ++v) s[v] = __builtin_fmaf(s[v], a.scale, sb[v]);
                     } else {
 #pragma unroll
+                        for (int t = 0; t < C::NKD; ++t) s = T::mfma(ka[t], qr[qb][t], s);
+#pragma unroll
                         for (int v = 0; v < 16; ++v) s[v] *= a.scale;
                     }
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], dp);
-                    const int query = wq0 + qb * 32 + c;
-                    if constexpr (C::MASK) {
-#pragma unroll
-                        for (int v = 0; v < 16; ++v)
-                            s[v] += dq_mask_at<T>(a.mask, mbase, query, n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3),
-                                                  a.Lq, a.Lk);
-                    }
                     const bool edge = (n0 + kb * 32 + 32 > a.Lk) || (a.causal && n0 + kb * 32 + 31 > wq0 + qb * 32);
                     if (edge) {
 #pragma unroll

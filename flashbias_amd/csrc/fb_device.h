@@ -89,6 +89,7 @@ struct MaskDesc {
     int64_t sb, sh, sm;
     int type;   // 0 none, 1 vector, 2 matrix
     int is_f32; // else same 16-bit type as the inputs
+    int vec_ok; // base and strides allow aligned loads of four consecutive keys
 };
 
 // Eight consecutive channels [col0, col0 + 8) of row `row` of a (rows x ncols) matrix with row
@@ -231,6 +232,65 @@ struct TileDma {
         }
     }
 };
+
+// Additive-mask values for the 16 scores that one lane holds of a 32 x 32 block, in C-layout
+// register order, as fp32.  They are used as the initial value of an accumulator (or as the
+// addend of the FMA that applies the softmax scale), so the mask costs no add per score.
+//
+// Lane = query (forward, dq kernel): register v <-> key k0 + 8 (v / 4) + 4 g + v % 4 of the
+// lane's own mask row `row` (byte pointer; the same row for every lane of a vector mask): four
+// runs of four consecutive keys, one aligned load each when the mask allows it.  Keys past Lk
+// read as 0 (their scores are set to -inf afterwards).
+template <class T>
+__device__ __forceinline__ void mask_block_keys(const MaskDesc &m, const uint8_t *row, int k0, int g, int Lk,
+                                                f32x16_t &out) {
+    if (m.vec_ok && k0 + 32 <= Lk) {
+        if (m.is_f32) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const f32x4_t x = *reinterpret_cast<const f32x4_t *>(row + (int64_t)(k0 + 8 * j + 4 * g) * 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) out[4 * j + e] = x[e];
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const u32x2_t x = *reinterpret_cast<const u32x2_t *>(row + (int64_t)(k0 + 8 * j + 4 * g) * 2);
+                out[4 * j + 0] = T::to_float((uint16_t)(x[0] & 0xffffu));
+                out[4 * j + 1] = T::to_float((uint16_t)(x[0] >> 16));
+                out[4 * j + 2] = T::to_float((uint16_t)(x[1] & 0xffffu));
+                out[4 * j + 3] = T::to_float((uint16_t)(x[1] >> 16));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 8 * (v >> 2) + 4 * g + (v & 3);
+            const int kc = key < Lk ? key : Lk - 1;
+            const float x = m.is_f32 ? reinterpret_cast<const float *>(row)[kc]
+                                     : T::to_float(reinterpret_cast<const uint16_t *>(row)[kc]);
+            out[v] = key < Lk ? x : 0.f;
+        }
+    }
+}
+
+// Lane = key (dk/dv kernel): register v <-> query q0 + 8 (v / 4) + 4 g + v % 4, all of key `key`:
+// sixteen element loads, consecutive lanes reading consecutive keys of a row.  `base` is the
+// byte pointer of the (batch, head) mask.  Out-of-range pairs read as 0.
+template <class T>
+__device__ __forceinline__ void mask_block_queries(const MaskDesc &m, const uint8_t *base, int q0, int g, int key, int Lq,
+                                                   int Lk, f32x16_t &out) {
+    const int kc = key < Lk ? key : Lk - 1;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int q = q0 + 8 * (v >> 2) + 4 * g + (v & 3);
+        const int qc = q < Lq ? q : Lq - 1;
+        const int64_t off = (m.type == 2 ? (int64_t)qc * m.sm : 0) + kc;
+        const float x = m.is_f32 ? reinterpret_cast<const float *>(base)[off]
+                                 : T::to_float(reinterpret_cast<const uint16_t *>(base)[off]);
+        out[v] = (q < Lq && key < Lk) ? x : 0.f;
+    }
+}
 
 // Grid id -> logical work id such that the workgroups that land on one XCD (hardware hands
 // consecutive ids to the 8 XCDs round-robin) cover a contiguous range of logical ids and so

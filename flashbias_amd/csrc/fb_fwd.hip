@@ -203,15 +203,6 @@ struct FwdLoader {
     }
 };
 
-// Additive mask value for (query, key); 0 outside the tensor (those scores are -inf anyway).
-template <class T>
-__device__ __forceinline__ float mask_at(const MaskDesc &m, const uint8_t *base, int query, int key, int Lq, int Lk) {
-    if (key >= Lk || query >= Lq) return 0.f;
-    const int64_t off = (m.type == 2 ? (int64_t)query * m.sm : 0) + key;
-    if (m.is_f32) return reinterpret_cast<const float *>(base)[off];
-    return T::to_float(reinterpret_cast<const uint16_t *>(base)[off]);
-}
-
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, C::WAVES_EU))) void fwd_kernel(
     const FwdArgs a) {
@@ -337,13 +328,25 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                 if (C::QB > 1 && a.causal && ns > bq0 + 31) continue;
                 // ---- S^T = [K | K_b] [scale Q | Q_b]^T
                 f32x16_t s[C::KBLK];
+                // additive mask: requested up front, it is the initial value of the bias chain
+                f32x16_t mk[C::MASK ? C::KBLK : 1];
+                if constexpr (C::MASK) {
+                    const uint8_t *mrow = mbase + (a.mask.type == 2 ? (int64_t)min(query, a.Lq - 1) * a.mask.sm : 0) *
+                                                      (a.mask.is_f32 ? 4 : 2);
+#pragma unroll
+                    for (int kb = 0; kb < C::KBLK; ++kb)
+                        mask_block_keys<T>(a.mask, mrow, ns + kb * 32, g, a.Lk, mk[kb]);
+                }
 #pragma unroll
                 for (int kb = 0; kb < C::KBLK; ++kb) {
                     // the q k^T part and the bias part are two independent MFMA chains, joined by
                     // one FMA per score that applies the softmax scale in fp32 (:246-256)
                     f32x16_t acc, accb;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[v] = accb[v] = 0.f;
+                    for (int v = 0; v < 16; ++v) {
+                        acc[v] = 0.f;
+                        accb[v] = C::MASK ? mk[C::MASK ? kb : 0][v] : 0.f;
+                    }
 #pragma unroll
                     for (int t = 0; t < C::NK; ++t) {
                         const u32x4_t kf = t < C::KPRE ? ka[kb][t < C::KPRE ? t : 0]
@@ -356,19 +359,10 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                     }
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
-                        acc[v] = C::NKR > 0 ? __builtin_fmaf(acc[v], a.scale, accb[v]) : acc[v] * a.scale;
+                        acc[v] = (C::NKR > 0 || C::MASK) ? __builtin_fmaf(acc[v], a.scale, accb[v]) : acc[v] * a.scale;
                     s[kb] = acc;
                 }
-                // ---- additive mask, then -inf for keys past the end and causal-hidden pairs
-                if constexpr (C::MASK) {
-#pragma unroll
-                    for (int kb = 0; kb < C::KBLK; ++kb)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int key = ns + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
-                            s[kb][v] += mask_at<T>(a.mask, mbase, query, key, a.Lq, a.Lk);
-                        }
-                }
+                // ---- -inf for keys past the end and causal-hidden pairs
                 const bool ragged = ns + C::BSUB > a.Lk;
                 const bool diag = a.causal && (ns + C::BSUB - 1 > bq0);
                 if (ragged || diag) {
