@@ -282,11 +282,28 @@ bwd_dkv_kernel(const BwdArgs a) {
     }
     __syncthreads();
 
+    // Additive mask: the values of a step (16 per lane and 32 x 32 block) are requested one step
+    // ahead and added by the FMA that applies the softmax scale.
+    f32x16_t mk[C::MASK ? C::QBLK : 1][C::MASK ? C::KBW : 1], mkn[C::MASK ? C::QBLK : 1][C::MASK ? C::KBW : 1];
+    auto load_mask = [&](f32x16_t (&dst)[C::MASK ? C::QBLK : 1][C::MASK ? C::KBW : 1], int m0) {
+#pragma unroll
+        for (int qb = 0; qb < C::QBLK; ++qb)
+#pragma unroll
+            for (int kb = 0; kb < C::KBW; ++kb)
+                mask_block_queries<T>(a.mask, mbase, m0 + qb * 32, g, wk0 + kb * 32 + c, a.Lq, a.Lk, dst[qb][kb]);
+    };
+    if constexpr (C::MASK) {
+        if (step0 < nsteps) load_mask(mk, step0 * C::BMQ);
+    }
+
     int cur = 0; // stage of the current step
     for (int step = step0; step < nsteps; ++step) {
         const int m0 = step * C::BMQ;
         const bool more = step + 1 < nsteps;
         const int nxt = cur == C::NSTAGE - 1 ? 0 : cur + 1;
+        if constexpr (C::MASK) {
+            if (more) load_mask(mkn, m0 + C::BMQ);
+        }
         if constexpr (C::VEC) {
             if (step + AHEAD < nsteps) {
                 const int tgt = nxt == C::NSTAGE - 1 ? 0 : nxt + 1; // the stage that step - 1 has left
@@ -330,9 +347,6 @@ bwd_dkv_kernel(const BwdArgs a) {
                             dp[4 * bq + e] = d4[e];
                         }
                     }
-                    // additive mask: requested before the MFMAs, added by the FMA that applies the scale
-                    f32x16_t mk;
-                    if constexpr (C::MASK) mask_block_queries<T>(a.mask, mbase, m0 + qb * 32, g, key, a.Lq, a.Lk, mk);
 #pragma unroll
                     for (int v = 0; v < 16; ++v) s[v] = 0.f;
 #pragma unroll
@@ -342,7 +356,8 @@ bwd_dkv_kernel(const BwdArgs a) {
                     // the softmax scale multiplies the fp32 q k^T accumulator before the bias steps
                     // (one chain keeps this kernel at three waves per SIMD)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mk[v]) : s[v] * a.scale;
+                    for (int v = 0; v < 16; ++v)
+                        s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mk[C::MASK ? qb : 0][C::MASK ? kb : 0][v]) : s[v] * a.scale;
 #pragma unroll
                     for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
                     const bool edge = (wk0 + kb * 32 + 32 > a.Lk) || (a.causal && wk0 + kb * 32 + 31 > m0 + qb * 32);
@@ -394,6 +409,12 @@ bwd_dkv_kernel(const BwdArgs a) {
             __syncthreads();
         }
         cur = nxt;
+        if constexpr (C::MASK) {
+#pragma unroll
+            for (int qb = 0; qb < C::QBLK; ++qb)
+#pragma unroll
+                for (int kb = 0; kb < C::KBW; ++kb) mk[qb][kb] = mkn[qb][kb];
+        }
     }
 
     // ---- epilogue: dv, dk (times scale), dk_bias for this lane's keys

@@ -281,6 +281,13 @@ template <class T>
 __device__ __forceinline__ void mask_block_queries(const MaskDesc &m, const uint8_t *base, int q0, int g, int key, int Lq,
                                                    int Lk, f32x16_t &out) {
     const int kc = key < Lk ? key : Lk - 1;
+    if (m.type == 1) { // vector mask: one value per key, i.e. per lane
+        const float x = m.is_f32 ? reinterpret_cast<const float *>(base)[kc]
+                                 : T::to_float(reinterpret_cast<const uint16_t *>(base)[kc]);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) out[v] = key < Lk ? x : 0.f;
+        return;
+    }
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
         const int q = q0 + 8 * (v >> 2) + 4 * g + (v & 3);
