@@ -26,6 +26,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
+# HBM bytes of one dk/dv launch at the headline shape: rocprofv3 FETCH_SIZE (x2.0, calibrated on a copy of
+# known size) + WRITE_SIZE, see profiles/headline_fwd_bwd_kernels.md; a counter figure, not measured live
+DKV_HBM_BYTES = 1.77e8
 PEAK_HBM_GBS = 8000.0
 
 
@@ -68,7 +71,7 @@ def _phase_timers(w, dev):
     from flashbias_amd.interface import _prepare, _stream, _tensor
     lib = _lib.load()
     q, k, v, qb, kb, do = (w[n] for n in ("q", "k", "v", "q_bias", "k_bias", "do"))
-    p, keep = _prepare(q, k, v, qb, kb, None, w["causal"], w["softmax_scale"])
+    p, keep = _prepare(q, k, v, qb, kb, w.get("mask"), w["causal"], w["softmax_scale"])
     o = torch.empty_like(q)
     lse = torch.empty((p.B, p.H, p.Lq), device=dev, dtype=torch.float32)
     p.o, p.lse = _tensor(o), lse.data_ptr()
@@ -167,7 +170,7 @@ def headline(args):
         "reference_formula_tflops": round(ref_fb / (ms_step * 1e-3) / 1e12, 2),
         "roofline": {"kernel": "bwd_dkv_kernel (fb_bwd_dkv)", "bound": "mfma", "achieved": round(tflops_main, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_main / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None},
+                     "traffic": DKV_HBM_BYTES},
     }
     del keep
     if not args.no_cpu:
@@ -221,7 +224,9 @@ def report(args):
     cases = [(f"sweep L={L}", lambda L=L: workloads.sweep(L), True) for L in workloads.SWEEP_LENGTHS]
     cases += [(f"alibi causal L={L}", lambda L=L: workloads.alibi(L), False) for L in (2048, 4096, 8192)]
     cases += [("swin 4096x256 r16", lambda: workloads.swin(), False), ("pde N=32768 r5", lambda: workloads.pde(), False),
-              ("pairformer 768 r32", lambda: workloads.pairformer(), False)]
+              ("pairformer 768 r32", lambda: workloads.pairformer(), False),
+              ("sweep L=4096 + vector mask", lambda: workloads.masked(4096, "vector"), None),
+              ("sweep L=4096 + matrix mask", lambda: workloads.masked(4096, "matrix"), None)]
     for name, make, dense in cases:
         w = _to_dev(make(), dev)
         B, Lq, H, d = w["q"].shape
@@ -233,8 +238,9 @@ def report(args):
         ours_fb = ours_fwd + ms["fb_bwd_preprocess"] + ms["fb_bwd_dkv"] + ms["fb_bwd_dq"]
         del keep
         leaves = [w[n].requires_grad_(True) for n in ("q", "k", "v", "q_bias", "k_bias")]
-        cat_fwd, cat_fb = _time_torch(lambda: _sdpa_concat(w), leaves, w["do"], args.steps, args.warmup)
-        den_fwd = den_fb = float("nan")
+        cat_fwd = cat_fb = den_fwd = den_fb = float("nan")
+        if dense is not None:  # the comparison providers are timed on the unmasked workloads only
+            cat_fwd, cat_fb = _time_torch(lambda: _sdpa_concat(w), leaves, w["do"], args.steps, args.warmup)
         if dense:
             with torch.no_grad():
                 bias = (w["q_bias"].permute(0, 2, 1, 3) @ w["k_bias"].permute(0, 2, 3, 1)).contiguous()

@@ -37,6 +37,16 @@ def sweep(L, B=2, H=4, d=32, r=8, dtype=torch.bfloat16, seed=0, causal=False):
     return _pack(q, k, v, do, qb, kb, causal, 1.0 / math.sqrt(d))
 
 
+def masked(L, kind, B=2, H=4, dtype=torch.bfloat16, seed=0):
+    """The sweep workload plus an additive mask: kind "vector" = (B, 1, 1, L) key-padding style,
+    kind "matrix" = (1, H, L, L) per-head matrix broadcast over the batch."""
+    w = sweep(L, B=B, H=H, dtype=dtype, seed=seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    shape = (B, 1, 1, L) if kind == "vector" else (1, H, L, L)
+    w["mask"] = torch.randn(*shape, generator=g).to(dtype)
+    return w
+
+
 def plumbing(seed=0):
     """fp32, non-causal, B2 H4 L1024 d32 r8 (CPU-runnable configuration)."""
     return sweep(1024, dtype=torch.float32, seed=seed)
