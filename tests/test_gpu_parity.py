@@ -177,6 +177,63 @@ def test_backward_reproducibility(gpu_device):
             assert torch.equal(runs[0][idx], other[idx])
 
 
+def test_backward_phases_through_the_c_abi(gpu_device):
+    """fb_bwd_preprocess / fb_bwd_dkv / fb_bwd_dq called one by one give what fb_bwd gives, and
+    the preprocess leaves -rowsum(o * dO) and lse * log2(e) in the scratch buffer (the delta of
+    flash_bias_triton.py:358-400 with the sign and the scaling that the main kernels consume)."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _prepare, _stream, _tensor
+    dev = gpu_device
+    B, L, H, d, r = 2, 333, 3, 32, 8
+    q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=11)]
+    lib = _lib.load()
+
+    def params():
+        p, keep = _prepare(q, k, v, qb, kb, None, True, None)
+        bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, L), device=dev, dtype=torch.float32),
+                    dq=torch.empty_like(q), dk=torch.empty_like(k), dv=torch.empty_like(v),
+                    dqb=torch.empty((B, L, H, r), device=dev, dtype=q.dtype),
+                    dkb=torch.empty((B, L, H, r), device=dev, dtype=q.dtype),
+                    scratch=torch.full((2, B, H, L), float("nan"), device=dev, dtype=torch.float32))
+        p.o, p.lse, p.dout = _tensor(bufs["o"]), bufs["lse"].data_ptr(), _tensor(do)
+        p.dq, p.dk, p.dv = _tensor(bufs["dq"]), _tensor(bufs["dk"]), _tensor(bufs["dv"])
+        p.dq_bias, p.dk_bias, p.delta = _tensor(bufs["dqb"]), _tensor(bufs["dkb"]), bufs["scratch"].data_ptr()
+        return p, keep, bufs
+
+    p1, keep1, whole = params()
+    _lib.check_status(lib.fb_fwd(p1, _stream()))
+    _lib.check_status(lib.fb_bwd(p1, _stream()))
+    p2, keep2, parts = params()
+    _lib.check_status(lib.fb_fwd(p2, _stream()))
+    for name in ("fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq"):
+        _lib.check_status(getattr(lib, name)(p2, _stream()))
+    torch.cuda.synchronize()
+    for name in ("o", "lse", "dq", "dk", "dv", "dqb", "dkb", "scratch"):
+        assert torch.equal(whole[name], parts[name]), name
+    o, lse = whole["o"].float(), whole["lse"]
+    delta = (o * do.float()).sum(-1).permute(0, 2, 1)  # (B, H, L)
+    assert torch.allclose(whole["scratch"][0], -delta, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(whole["scratch"][1], lse * math.log2(math.e), rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.parametrize("Lq,Lk", [(1000, 1000), (777, 1300), (1300, 777)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_long_ragged_sequences(gpu_device, Lq, Lk, causal):
+    """Many steps through the three-stage LDS ring of the dk/dv kernel, last step ragged."""
+    _case(gpu_device, 1, Lq, Lk, 2, 32, 8, torch.bfloat16, causal, seed=12)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("offset", [0, 1])
+def test_matrix_mask_alignment(gpu_device, dtype, offset):
+    """Matrix masks that allow aligned 4-key loads, and views of them that do not."""
+    B, L, H = 1, 200, 2
+    g = torch.Generator().manual_seed(13)
+    big = torch.randn(1, H, L, L + 8, generator=g).to(dtype)
+    mask = big[..., offset:offset + L]  # row stride L + 8; offset 1 breaks the alignment of every row
+    _case(gpu_device, B, L, L, H, 32, 8, torch.bfloat16, False, mask=mask, seed=14)
+
+
 # ------------------------------------------------------------------ named workloads (reduced)
 def _run_workload(gpu_device, w, dtype, skip=()):
     ref = oracle(w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], None, w["causal"], w["softmax_scale"], w["do"])
