@@ -47,7 +47,7 @@ struct DkvCfg {
     static constexpr int CQ = 2 * NKD, CR = 2 * NKR, CO = 2 * NKD;
     static constexpr int TASKS = BMQ * (CQ + CR + CO);
     static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
-    static constexpr int WAVES_EU = (NK <= 4 && NDV <= 2) ? 2 : 1;
+    static constexpr int WAVES_EU = (NK <= 6 && NDV <= 2) ? 2 : 1;
 };
 
 template <class C>

@@ -28,7 +28,7 @@ struct DqCfg {
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dQ | dQ_b]^T
-    static constexpr int QBLK = (NK <= 4 && !MASK_) ? 2 : 1; // the mask values need the registers of the second block
+    static constexpr int QBLK = (NK <= 3 && !MASK_) ? 2 : 1; // the mask values need the registers of the second block
     static constexpr int BM = NWAVES * QBLK * 32;
     static constexpr int KBLK = 2, BN = 32 * KBLK;
     // sK row: [K | K_b] of one key in ROWCH swizzled 16-byte chunks; the one copy is read
@@ -43,7 +43,7 @@ struct DqCfg {
     static constexpr int K_TASKS = BN * (CD + CR), V_TASKS = BN * CD;
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
-    static constexpr int WAVES_EU = (NK <= 4) ? 2 : 1;
+    static constexpr int WAVES_EU = (NK <= 6) ? 2 : 1;
 };
 
 template <class C>

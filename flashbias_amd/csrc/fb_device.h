@@ -133,12 +133,16 @@ __device__ __forceinline__ int slot_of(int x) {
 // rows = tile rows) and column-wise (ds_read_b64_tr_b16: A operand with rows = tile columns)
 // keep one row-major copy whose 16-byte chunks are XOR-swizzled by row, so that both access
 // patterns are free of bank conflicts.  ROWCH = chunks per row (8 -> 128-byte rows).
-__device__ __forceinline__ int swz_of(int row) { // 3-bit chunk swizzle from row bits 1, 2, 3
-    return ((row & 2) << 1) | ((row >> 2) & 1) | ((row >> 2) & 2);
+template <int ROWCH>
+__device__ __forceinline__ int swz_of(int row) {
+    // 128-byte rows: row bit 0 already selects the bank half, bits 1, 2, 3 swizzle three chunk
+    // bits; longer rows are a multiple of all 64 banks, so bit 0 swizzles a fourth chunk bit
+    const int s3 = ((row & 2) << 1) | ((row >> 2) & 1) | ((row >> 2) & 2);
+    return ROWCH == 8 ? s3 : s3 | ((row & 1) << 3);
 }
 template <int ROWCH>
 __device__ __forceinline__ int swz_off(int row, int chunk) { // element offset of a chunk
-    return (row * ROWCH + (chunk ^ swz_of(row))) * 8;
+    return (row * ROWCH + (chunk ^ swz_of<ROWCH>(row))) * 8;
 }
 
 // Transposing LDS read.  Within each group of 16 lanes, lane 4a + b receives as element j the
@@ -212,7 +216,7 @@ struct TileDma {
         for (int j = 0; j < NI; ++j) {
             const int p = (wave * NI + j) * 64 + lane;
             const int r = p / ROWCH, pos = p % ROWCH;
-            const int chunk = pos ^ swz_of(r);
+            const int chunk = pos ^ swz_of<ROWCH>(r);
             const bool is_b = chunk >= split;
             const int cc = is_b ? chunk - split : chunk;
             row[j] = r;
