@@ -198,7 +198,9 @@ __device__ __forceinline__ void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(
 // instruction fills 64 consecutive chunk positions of the tile and each lane fetches the global
 // chunk that the swizzle puts at its position.  Lanes whose position is channel padding stay
 // switched off (those chunks keep the zeros of the initial clear); rows past the end of the
-// tensor re-read its last row.  The NWAVES waves of the workgroup issue equal shares.
+// tensor re-read its last row.  The NWAVES waves of the workgroup issue equal shares.  Every copy
+// instruction has active lanes (each tile row starts with a valid chunk, ncols_a >= 8), so a
+// wave always issues exactly NI of them per tile: the kernels' vmcnt waits count on that.
 template <int ROWS, int ROWCH, int NWAVES>
 struct TileDma {
     static constexpr int NI = ROWS * ROWCH / 64 / NWAVES; // copy instructions per wave
