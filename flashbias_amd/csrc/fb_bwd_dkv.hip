@@ -40,8 +40,15 @@ struct DkvCfg {
     static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
     static constexpr int ROWCHO = 2 * NKD <= 8 ? 8 : 16;
     static constexpr int SQ = BMQ * ROWCH * 8, SDO = BMQ * ROWCHO * 8;
-    static constexpr int STAGE_ELEMS = SQ + SDO + 4 * BMQ; // + lse * log2(e), -delta as fp32
-    static constexpr int NSTAGE = 3;
+    // masked, aligned instantiations also stage the step's 64 x 128 tile of a 16-bit matrix mask
+    static constexpr bool MTILE = VEC_ && MASK_;
+    static constexpr int MROWCH = BN / 8; // chunks per mask-tile row
+    static constexpr int SM = MTILE ? BMQ * BN : 0;
+    static constexpr int STAGE_ELEMS = SQ + SDO + 4 * BMQ + SM; // + lse * log2(e), -delta as fp32
+    // direct loader: three stages, two steps ahead; with a mask tile (or the element-wise loader) two
+    // stages, one step ahead
+    static constexpr int AHEAD = (VEC_ && !MASK_) ? 2 : 1;
+    static constexpr int NSTAGE = AHEAD + 1;
     static constexpr int LDS_BYTES = NSTAGE * STAGE_ELEMS * 2;
     // loader tasks: 8-channel chunks of Q, Q_b and dout, one query row each
     static constexpr int CQ = 2 * NKD, CR = 2 * NKR, CO = 2 * NKD;
@@ -140,6 +147,8 @@ template <class C>
 struct DkvDirect {
     TileDma<C::BMQ, C::ROWCH, C::NWAVES> q;
     TileDma<C::BMQ, C::ROWCHO, C::NWAVES> d;
+    TileDma<C::BMQ, C::MROWCH, C::NWAVES> m; // mask tile (masked instantiations, 16-bit matrix masks)
+    bool mtile;
     static constexpr int N = decltype(q)::NI + decltype(d)::NI;
     // waves 0 and 1 also fetch the step's lse * log2(e) and -delta rows (BMQ = 64 floats: one
     // 4-byte copy per lane)
@@ -156,6 +165,14 @@ struct DkvDirect {
         stat = wave == 0 ? lse2 : wave == 1 ? negd : nullptr;
         q.init(qbase, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? qbbase : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane);
         d.init(dobase, a.dout.ss, a.d, C::ROWCHO, nullptr, 0, 0, wave, lane);
+        mtile = false;
+    }
+
+    // The workgroup's columns [n0, n0 + BN) of the (batch, head) mask matrix, 16-bit elements.
+    __device__ __forceinline__ void init_mask(const BwdArgs &a, const uint8_t *mbase, int n0) {
+        mtile = true;
+        const int ncols = a.Lk - n0 < C::BN ? a.Lk - n0 : C::BN;
+        m.init(reinterpret_cast<const uint16_t *>(mbase) + n0, a.mask.sm, ncols, C::MROWCH, nullptr, 0, 0, wave, lane);
     }
 
     __device__ __forceinline__ void issue(uint16_t *stage, int m0, int Lq) const {
@@ -163,6 +180,9 @@ struct DkvDirect {
         q.issue(base, m0, Lq);
         d.issue(base + 2 * C::SQ, m0, Lq);
         if (wave < 2) lds_dma4(stat + min(m0 + lane, Lq - 1), base + 2 * (C::SQ + C::SDO) + wave * (4 * C::BMQ));
+        if constexpr (C::MTILE) {
+            if (mtile) m.issue(base + 2 * (C::SQ + C::SDO + 4 * C::BMQ), m0, Lq);
+        }
     }
 
     // Loads of this wave that may stay in flight when the data of the step before them is needed.
@@ -259,18 +279,25 @@ bwd_dkv_kernel(const BwdArgs a) {
         for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
     }
     __syncthreads();
-    // Step s is computed from stage (s - step0) % 3.  Direct loader: the tiles of step s + 2 are
-    // requested at the top of step s; element-wise loader: step s + 1 goes through registers.
-    constexpr int AHEAD = C::VEC ? 2 : 1;
+    // Step s is computed from stage (s - step0) % NSTAGE.  Direct loader: the tiles of step
+    // s + AHEAD are requested at the top of step s; element-wise loader: step s + 1 goes through
+    // registers.
+    constexpr int AHEAD = C::AHEAD;
     DkvDirect<C> direct;
     DkvStage<C> st;
     if constexpr (C::VEC) {
         direct.init(a, qbase, qbbase, dobase, lse2, negd, wave, lane);
+        if constexpr (C::MTILE) {
+            // a 16-bit matrix mask whose rows allow 16-byte copies goes through the LDS stages
+            if (a.mask.type == 2 && a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 &&
+                reinterpret_cast<uintptr_t>(mbase) % 16 == 0)
+                direct.init_mask(a, mbase, n0);
+        }
 #pragma unroll
         for (int k = 0; k < AHEAD; ++k)
             if (step0 + k < nsteps) direct.issue(stage0 + k * C::STAGE_ELEMS, (step0 + k) * C::BMQ, a.Lq);
         // the first step's tiles must have landed; the second step's may still be in flight
-        if (step0 + 1 < nsteps)
+        if (AHEAD == 2 && step0 + 1 < nsteps)
             direct.template wait_older<true>();
         else
             direct.template wait_older<false>();
@@ -292,8 +319,9 @@ bwd_dkv_kernel(const BwdArgs a) {
             for (int kb = 0; kb < C::KBW; ++kb)
                 mask_block_queries<T>(a.mask, mbase, m0 + qb * 32, g, wk0 + kb * 32 + c, a.Lq, a.Lk, dst[qb][kb]);
     };
+    const bool mtile = C::MTILE && direct.mtile; // else the mask values travel through registers
     if constexpr (C::MASK) {
-        if (step0 < nsteps) load_mask(mk, step0 * C::BMQ);
+        if (step0 < nsteps && !mtile) load_mask(mk, step0 * C::BMQ);
     }
 
     int cur = 0; // stage of the current step
@@ -302,11 +330,11 @@ bwd_dkv_kernel(const BwdArgs a) {
         const bool more = step + 1 < nsteps;
         const int nxt = cur == C::NSTAGE - 1 ? 0 : cur + 1;
         if constexpr (C::MASK) {
-            if (more) load_mask(mkn, m0 + C::BMQ);
+            if (more && !mtile) load_mask(mkn, m0 + C::BMQ);
         }
         if constexpr (C::VEC) {
             if (step + AHEAD < nsteps) {
-                const int tgt = nxt == C::NSTAGE - 1 ? 0 : nxt + 1; // the stage that step - 1 has left
+                const int tgt = (cur + AHEAD) % C::NSTAGE; // the stage that step - 1 has left
                 direct.issue(stage0 + tgt * C::STAGE_ELEMS, m0 + AHEAD * C::BMQ, a.Lq);
             }
             direct.fix_ragged(stage0 + cur * C::STAGE_ELEMS, m0, a.Lq, tid);
@@ -317,6 +345,7 @@ bwd_dkv_kernel(const BwdArgs a) {
         const uint16_t *sQ = stage0 + cur * C::STAGE_ELEMS;
         const uint16_t *sdO = sQ + C::SQ;
         const float *sStat = reinterpret_cast<const float *>(sdO + C::SDO);
+        const uint16_t *sM = sdO + C::SDO + 4 * C::BMQ;
 
         const bool visible = !(a.causal && wk0 > m0 + C::BMQ - 1) && wk0 < a.Lk;
         if (visible) {
@@ -353,11 +382,30 @@ bwd_dkv_kernel(const BwdArgs a) {
                     for (int t = 0; t < C::NKD; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(da[t], vreg[kb][t], dp);
+                    f32x16_t mval; // additive mask of this block, added by the FMA that applies the scale
+                    if constexpr (C::MASK) {
+                        if (mtile) { // column `key`, rows in C-layout order: four transposing reads
+                            if constexpr (C::MTILE) {
+                                const int col = (wave * C::KBW + kb) * 32 + 16 * (c >> 4) + 4 * (c & 3);
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const int row = qb * 32 + 8 * j + 4 * g + ((c & 15) >> 2);
+                                    const u32x2_t x = lds_read_tr4(sM + swz_off<C::MROWCH>(row, col >> 3) + (col & 7));
+                                    mval[4 * j + 0] = T::to_float((uint16_t)(x[0] & 0xffffu));
+                                    mval[4 * j + 1] = T::to_float((uint16_t)(x[0] >> 16));
+                                    mval[4 * j + 2] = T::to_float((uint16_t)(x[1] & 0xffffu));
+                                    mval[4 * j + 3] = T::to_float((uint16_t)(x[1] >> 16));
+                                }
+                            }
+                        } else {
+                            mval = mk[C::MASK ? qb : 0][C::MASK ? kb : 0];
+                        }
+                    }
                     // the softmax scale multiplies the fp32 q k^T accumulator before the bias steps
                     // (one chain keeps this kernel at three waves per SIMD)
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
-                        s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mk[C::MASK ? qb : 0][C::MASK ? kb : 0][v]) : s[v] * a.scale;
+                        s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mval[v]) : s[v] * a.scale;
 #pragma unroll
                     for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
                     const bool edge = (wk0 + kb * 32 + 32 > a.Lk) || (a.causal && wk0 + kb * 32 + 31 > m0 + qb * 32);
@@ -396,7 +444,7 @@ bwd_dkv_kernel(const BwdArgs a) {
         }
         if constexpr (C::VEC) {
             // the next step's tiles must have landed; the one after may still be in flight
-            if (step + AHEAD < nsteps)
+            if (AHEAD == 2 && step + AHEAD < nsteps)
                 direct.template wait_older<true>();
             else
                 direct.template wait_older<false>();
