@@ -43,11 +43,6 @@ struct BF16 {
     static __device__ __forceinline__ uint16_t from_float(float x) {
         return __builtin_bit_cast(uint16_t, (__bf16)x);
     }
-    // acc + lo(x) + hi(x) for a packed pair
-    static __device__ __forceinline__ float dot2_ones(uint32_t x, float acc) {
-        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x),
-                                               __builtin_bit_cast(bf16x2_t, 0x3f803f80u), acc, false);
-    }
     static constexpr uint16_t kOne = 0x3f80;
 };
 
@@ -68,10 +63,6 @@ struct F16 {
     }
     static __device__ __forceinline__ uint16_t from_float(float x) {
         return __builtin_bit_cast(uint16_t, (_Float16)x);
-    }
-    static __device__ __forceinline__ float dot2_ones(uint32_t x, float acc) {
-        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, x), __builtin_bit_cast(f16x2_t, 0x3c003c00u), acc,
-                                      false);
     }
     static constexpr uint16_t kOne = 0x3c00;
 };
@@ -324,19 +315,5 @@ __device__ __forceinline__ float half_wave_max(float x) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// scale * x for the eight 16-bit values of a chunk, as hi + lo parts in the same 16-bit type
-// (hi = round(scale x), lo = round(scale x - hi)): 16 mantissa bits of the scaled value.
-template <class T>
-__device__ __forceinline__ void split_scaled(const u32x4_t x, float scale, u32x4_t &hi, u32x4_t &lo) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float a = T::to_float((uint16_t)(x[i] & 0xffffu)) * scale;
-        const float b = T::to_float((uint16_t)(x[i] >> 16)) * scale;
-        hi[i] = T::pack2(a, b);
-        const float ah = T::to_float((uint16_t)(hi[i] & 0xffffu)), bh = T::to_float((uint16_t)(hi[i] >> 16));
-        lo[i] = T::pack2(a - ah, b - bh);
-    }
-}
 
 } // namespace fb
