@@ -234,6 +234,43 @@ def test_matrix_mask_alignment(gpu_device, dtype, offset):
     _case(gpu_device, B, L, L, H, 32, 8, torch.bfloat16, False, mask=mask, seed=14)
 
 
+def _random_case(idx):
+    """A reproducible draw from the space of supported shapes: lengths, head dim, rank, dtype,
+    causal flag, factor broadcasting and mask kind / dtype / alignment."""
+    import random
+    rnd = random.Random(1000 + idx)
+    d = rnd.choice([8, 16, 24, 32, 32, 32, 40, 64, 64, 72, 128])
+    r = rnd.choice([0, 8, 8, 8, 16, 24, 32, 64])
+    lens = [rnd.choice([1, 17, 63, 64, 65, 127, 128, 129, 200, 256, 333, 512, 640, 701]) for _ in range(2)]
+    if rnd.random() < 0.5:
+        lens[1] = lens[0]
+    dtype = rnd.choice([torch.bfloat16, torch.float16])
+    causal = rnd.random() < 0.4
+    bq = (rnd.random() < 0.25, rnd.random() < 0.25)
+    bk = (rnd.random() < 0.25, rnd.random() < 0.25)
+    mask_kind = rnd.choice([None, None, "vector", "matrix", "matrix", "matrix_f32", "matrix_shifted"])
+    return dict(B=rnd.choice([1, 2]), H=rnd.choice([1, 3]), Lq=lens[0], Lk=lens[1], d=d, r=r, dtype=dtype, causal=causal,
+                bq=bq, bk=bk, mask_kind=mask_kind, scale=rnd.choice([None, 0.3]))
+
+
+@pytest.mark.parametrize("idx", range(40))
+def test_random_shapes(gpu_device, idx):
+    c = _random_case(idx)
+    g = torch.Generator().manual_seed(2000 + idx)
+    B, H, Lq, Lk = c["B"], c["H"], c["Lq"], c["Lk"]
+    mask = None
+    if c["mask_kind"] == "vector":
+        mask = torch.randn(B, 1, 1, Lk, generator=g).to(c["dtype"])
+    elif c["mask_kind"] == "matrix":
+        mask = torch.randn(1, H, Lq, Lk, generator=g).to(c["dtype"])
+    elif c["mask_kind"] == "matrix_f32":
+        mask = torch.randn(B, 1, Lq, Lk, generator=g)
+    elif c["mask_kind"] == "matrix_shifted":  # rows that are not 16-byte aligned
+        mask = torch.randn(1, H, Lq, Lk + 3, generator=g).to(c["dtype"])[..., 3:]
+    _case(gpu_device, B, Lq, Lk, H, c["d"], c["r"], c["dtype"], c["causal"], mask=mask, scale=c["scale"], seed=3000 + idx,
+          bq=c["bq"], bk=c["bk"])
+
+
 # ------------------------------------------------------------------ named workloads (reduced)
 def _run_workload(gpu_device, w, dtype, skip=()):
     ref = oracle(w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], None, w["causal"], w["softmax_scale"], w["do"])
