@@ -34,10 +34,13 @@ struct DqCfg {
     // sK row: [K | K_b] of one key in ROWCH swizzled 16-byte chunks; the one copy is read
     // row-wise for S^T and column-wise for [dQ | dQ_b]^T
     static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
-    static constexpr int DVP = 16 * NKD + 8; // sV row: V of one key
-    static constexpr int SK = BN * ROWCH * 8, SV = BN * DVP;
+    static constexpr int ROWCHV = 2 * NKD <= 8 ? 8 : 16; // sV row: V of one key, same chunk swizzle
+    static constexpr int SK = BN * ROWCH * 8, SV = BN * ROWCHV * 8;
     static constexpr int STAGE = SK + SV;
-    static constexpr int LDS_BYTES = 2 * STAGE * 2;
+    // direct loader: three stages, two tiles ahead; element-wise loader: two stages, one ahead
+    static constexpr int AHEAD = VEC_ ? 2 : 1;
+    static constexpr int NSTAGE = AHEAD + 1;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE * 2;
     // loader: 8-channel chunks of K, K_b and V, one key row each
     static constexpr int CD = 2 * NKD, CR = 2 * NKR;
     static constexpr int K_TASKS = BN * (CD + CR), V_TASKS = BN * CD;
@@ -47,11 +50,13 @@ struct DqCfg {
 };
 
 template <class C>
-struct DqStage {
-    u32x4_t k[C::K_PT];
-    u32x4_t v[C::V_PT];
+struct DqStage { // register staging of one tile, used by the element-wise loader only
+    u32x4_t k[C::VEC ? 1 : C::K_PT];
+    u32x4_t v[C::VEC ? 1 : C::V_PT];
 };
 
+// Element-wise loader (tensors that are not 16-byte aligned, d or r not a multiple of 8):
+// clamped loads into registers, written to LDS after the tile's arithmetic.
 template <class C>
 struct DqLoader {
     // K task: one key row x one 8-channel chunk of K (chunk < CD) or K_b
@@ -65,7 +70,7 @@ struct DqLoader {
     __device__ static __forceinline__ void load(DqStage<C> &st, const BwdArgs &a, const uint16_t *kbase,
                                                 const uint16_t *kbbase, const uint16_t *vbase, int n0, int tid) {
 #pragma unroll
-        for (int i = 0; i < C::K_PT; ++i) {
+        for (int i = 0; i < (C::VEC ? 1 : C::K_PT); ++i) {
             const int task = tid + i * C::NTHREADS;
             int row, ch;
             bool is_b;
@@ -75,83 +80,56 @@ struct DqLoader {
             const int ncols = is_b ? a.r : a.d;
             st.k[i] = u32x4_t{0u, 0u, 0u, 0u};
             if (C::K_TASKS % C::NTHREADS == 0 || task < C::K_TASKS)
-                st.k[i] = load_chunk<C::VEC>(base, ld, n0 + row, a.Lk, ch * 8, ncols);
+                st.k[i] = load_chunk<false>(base, ld, n0 + row, a.Lk, ch * 8, ncols);
         }
 #pragma unroll
-        for (int i = 0; i < C::V_PT; ++i) {
+        for (int i = 0; i < (C::VEC ? 1 : C::V_PT); ++i) {
             const int task = tid + i * C::NTHREADS;
             st.v[i] = u32x4_t{0u, 0u, 0u, 0u};
             if (C::V_TASKS % C::NTHREADS == 0 || task < C::V_TASKS)
-                st.v[i] = load_chunk<C::VEC>(vbase, a.v.ss, n0 + task % C::BN, a.Lk, (task / C::BN) * 8, a.d);
+                st.v[i] = load_chunk<false>(vbase, a.v.ss, n0 + task % C::BN, a.Lk, (task / C::BN) * 8, a.d);
         }
     }
 
-    __device__ static __forceinline__ void store(const DqStage<C> &st, uint16_t *stage, int tid,
-                                                 const bool (&kok)[C::K_PT], const bool (&vok)[C::V_PT]) {
+    // chunks in the zero padding of the channel dimension are never written (LDS cleared once)
+    __device__ static __forceinline__ void store(const DqStage<C> &st, const BwdArgs &a, uint16_t *stage, int tid) {
         uint16_t *sK = stage, *sV = sK + C::SK;
 #pragma unroll
-        for (int i = 0; i < C::K_PT; ++i) {
+        for (int i = 0; i < (C::VEC ? 1 : C::K_PT); ++i) {
             const int task = tid + i * C::NTHREADS;
             int row, ch;
             bool is_b;
             ktask(task, row, ch, is_b);
-            if (kok[i])
+            if (task < C::K_TASKS && ch * 8 < (is_b ? a.r : a.d))
                 *reinterpret_cast<u32x4_t *>(sK + swz_off<C::ROWCH>(row, (is_b ? 2 * C::NKD : 0) + ch)) = st.k[i];
         }
 #pragma unroll
-        for (int i = 0; i < C::V_PT; ++i) {
+        for (int i = 0; i < (C::VEC ? 1 : C::V_PT); ++i) {
             const int task = tid + i * C::NTHREADS;
-            if (vok[i]) *reinterpret_cast<u32x4_t *>(sV + (task % C::BN) * C::DVP + (task / C::BN) * 8) = st.v[i];
+            if (task < C::V_TASKS && (task / C::BN) * 8 < a.d)
+                *reinterpret_cast<u32x4_t *>(sV + swz_off<C::ROWCHV>(task % C::BN, task / C::BN)) = st.v[i];
         }
     }
 };
 
-// Per-thread constants of the fast loader (tiles entirely inside the sequence): running global
-// pointers advanced by one key tile at a time, plain loads that stay in flight during the
-// tile's arithmetic.  Chunks that lie in the zero padding of the channel dimension are never
-// stored (the LDS buffers are cleared once).
+// Direct loader (16-byte aligned tensors, d and r multiples of 8): the [K | K_b] and V tiles of
+// a key tile, copied straight into an LDS stage.
 template <class C>
-struct DqFast {
-    const uint16_t *kptr[C::K_PT], *vptr[C::V_PT];
-    int64_t kinc[C::K_PT], vinc[C::V_PT];
-    bool kok[C::K_PT], vok[C::V_PT];
+struct DqDirect {
+    TileDma<C::BN, C::ROWCH, C::NWAVES> k;
+    TileDma<C::BN, C::ROWCHV, C::NWAVES> v;
+    static constexpr int N = decltype(k)::NI + decltype(v)::NI;
 
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *kbase, const uint16_t *kbbase,
-                                         const uint16_t *vbase, int n0, int tid) {
-#pragma unroll
-        for (int i = 0; i < C::K_PT; ++i) {
-            const int task = tid + i * C::NTHREADS;
-            int row, ch;
-            bool is_b;
-            DqLoader<C>::ktask(task, row, ch, is_b);
-            const uint16_t *base = is_b ? kbbase : kbase;
-            const int64_t ld = is_b ? a.kb.ss : a.k.ss;
-            kok[i] = task < C::K_TASKS && ch * 8 < (is_b ? a.r : a.d);
-            kinc[i] = kok[i] ? ld * C::BN : 0;
-            kptr[i] = kok[i] ? base + (int64_t)(n0 + row) * ld + ch * 8 : kbase;
-        }
-#pragma unroll
-        for (int i = 0; i < C::V_PT; ++i) {
-            const int task = tid + i * C::NTHREADS;
-            const int row = task % C::BN, ch = task / C::BN;
-            vok[i] = task < C::V_TASKS && ch * 8 < a.d;
-            vinc[i] = vok[i] ? a.v.ss * C::BN : 0;
-            vptr[i] = vok[i] ? vbase + (int64_t)(n0 + row) * a.v.ss + ch * 8 : vbase;
-        }
+                                         const uint16_t *vbase, int wave, int lane) {
+        k.init(kbase, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? kbbase : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane);
+        v.init(vbase, a.v.ss, a.d, C::ROWCHV, nullptr, 0, 0, wave, lane);
     }
 
-    __device__ __forceinline__ void load(DqStage<C> &st) const {
-#pragma unroll
-        for (int i = 0; i < C::K_PT; ++i) st.k[i] = *reinterpret_cast<const u32x4_t *>(kptr[i]);
-#pragma unroll
-        for (int i = 0; i < C::V_PT; ++i) st.v[i] = *reinterpret_cast<const u32x4_t *>(vptr[i]);
-    }
-
-    __device__ __forceinline__ void advance() {
-#pragma unroll
-        for (int i = 0; i < C::K_PT; ++i) kptr[i] += kinc[i];
-#pragma unroll
-        for (int i = 0; i < C::V_PT; ++i) vptr[i] += vinc[i];
+    __device__ __forceinline__ void issue(uint16_t *stage, int n0, int Lk) const {
+        const uint32_t base = lds_addr_of(stage);
+        k.issue(base, n0, Lk);
+        v.issue(base + 2 * C::SK, n0, Lk);
     }
 };
 
@@ -221,28 +199,42 @@ bwd_dq_kernel(const BwdArgs a) {
     if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
     const int ntiles_k = (k_end + C::BN - 1) / C::BN;
 
-    {   // clear both LDS buffers once: the zero padding of the channel dimension is never rewritten
+    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
         u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
         for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
     }
     __syncthreads();
-    DqFast<C> fast;
-    fast.init(a, kbase, kbbase, vbase, C::BN, tid); // the first prefetch is tile 1
+    // Tile t is computed from stage t % NSTAGE.  Direct loader: tile t + 2 is requested at the top
+    // of tile t; element-wise loader: tile t + 1 goes through registers.  Keys past the end of a
+    // ragged last tile hold copies of the last key; their scores are set to -inf below.
+    constexpr int AHEAD = C::AHEAD;
+    DqDirect<C> direct;
     DqStage<C> st;
-    DqLoader<C>::load(st, a, kbase, kbbase, vbase, 0, tid);
-    DqLoader<C>::store(st, stage0, tid, fast.kok, fast.vok);
+    if constexpr (C::VEC) {
+        direct.init(a, kbase, kbbase, vbase, wave, lane);
+#pragma unroll
+        for (int k = 0; k < AHEAD; ++k)
+            if (k < ntiles_k) direct.issue(stage0 + k * C::STAGE, k * C::BN, a.Lk);
+        if (1 < ntiles_k)
+            wait_vmcnt<DqDirect<C>::N>(); // the first tile has landed, the second may be in flight
+        else
+            wait_vmcnt<0>();
+    } else {
+        DqLoader<C>::load(st, a, kbase, kbbase, vbase, 0, tid);
+        DqLoader<C>::store(st, a, stage0, tid);
+    }
     __syncthreads();
 
+    int cur = 0; // stage of the current tile
     for (int it = 0; it < ntiles_k; ++it) {
-        const int cur = it & 1;
         const int n0 = it * C::BN;
         const bool more = it + 1 < ntiles_k;
-        if (more) {
-            if (C::VEC && n0 + 2 * C::BN <= a.Lk)
-                fast.load(st);
-            else
-                DqLoader<C>::load(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
-            fast.advance();
+        const int nxt = cur == C::NSTAGE - 1 ? 0 : cur + 1;
+        if constexpr (C::VEC) {
+            if (it + AHEAD < ntiles_k)
+                direct.issue(stage0 + ((cur + AHEAD) % C::NSTAGE) * C::STAGE, n0 + AHEAD * C::BN, a.Lk);
+        } else if (more) {
+            DqLoader<C>::load(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
         }
 
         const uint16_t *sK = stage0 + cur * C::STAGE, *sV = sK + C::SK;
@@ -256,7 +248,7 @@ bwd_dq_kernel(const BwdArgs a) {
                     ka[t] = *reinterpret_cast<const u32x4_t *>(sK + swz_off<C::ROWCH>(kb * 32 + c, 2 * t + g));
 #pragma unroll
                 for (int t = 0; t < C::NKD; ++t)
-                    va[t] = *reinterpret_cast<const u32x4_t *>(sV + (kb * 32 + c) * C::DVP + 16 * t + 8 * g);
+                    va[t] = *reinterpret_cast<const u32x4_t *>(sV + swz_off<C::ROWCHV>(kb * 32 + c, 2 * t + g));
                 u32x4_t dsp[C::QBLK][2]; // dS^T, packed, per 16-key step
 #pragma unroll
                 for (int qb = 0; qb < C::QBLK; ++qb) {
@@ -318,8 +310,17 @@ bwd_dq_kernel(const BwdArgs a) {
                     }
             }
         }
-        if (more) DqLoader<C>::store(st, stage0 + (cur ^ 1) * C::STAGE, tid, fast.kok, fast.vok);
-        __syncthreads();
+        if constexpr (C::VEC) {
+            if (it + AHEAD < ntiles_k)
+                wait_vmcnt<DqDirect<C>::N>(); // the next tile has landed, the one after may be in flight
+            else
+                wait_vmcnt<0>();
+            barrier_lds();
+        } else {
+            if (more) DqLoader<C>::store(st, a, stage0 + nxt * C::STAGE, tid);
+            __syncthreads();
+        }
+        cur = nxt;
     }
 
     // ---- epilogue: dq = scale * acc rows [0, d), dq_bias = acc rows [16 NKD, 16 NKD + r)
