@@ -10,7 +10,7 @@
 //   S^T  = [K | K_b] [scale Q | Q_b]^T        A = key rows (LDS),        B = query registers
 //   dP^T = V dO^T                             A = value rows (LDS),      B = dO registers
 //   P^T  = exp(S^T - lse)                     lse is a per-lane scalar
-//   dS^T = P^T * (dP^T - delta)               delta is a per-lane scalar
+//   dS^T = P^T * (dP^T - delta)               -delta is the initial value of the dP^T accumulator
 //   [dQ | dQ_b]^T += [K | K_b]^T dS^T         A = key tile read column-wise (LDS), B = dS^T registers
 //
 // so dS^T goes from the accumulator layout straight into the next MFMA and [dQ | dQ_b]^T stays
@@ -169,7 +169,10 @@ bwd_dq_kernel(const BwdArgs a) {
     // ---- query-side operands, resident in registers
     u32x4_t qr[C::QBLK][C::NKD], qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
     u32x4_t dor[C::QBLK][C::NKD];
-    float negd[C::QBLK], lse2[C::QBLK]; // -delta and lse * log2(e) of this lane's queries
+    float lse2[C::QBLK]; // lse * log2(e) of this lane's queries
+    // -delta of this lane's query in all 16 registers of an accumulator block: the initial value
+    // of every dP^T chain (lane = query, so it is the same for every key), no add per score
+    f32x16_t negd[C::QBLK];
     f32x16_t acc[C::QBLK][C::MB];
 #pragma unroll
     for (int qb = 0; qb < C::QBLK; ++qb) {
@@ -188,7 +191,9 @@ bwd_dq_kernel(const BwdArgs a) {
         const int64_t sidx = (int64_t)bh * a.Lq + (ok ? query : a.Lq - 1);
         // the preprocess step left -delta and lse * log2(e) in the scratch buffer
         lse2[qb] = ok ? a.delta[(int64_t)a.B * a.H * a.Lq + sidx] : INFINITY; // rows past the end: P = exp2(-inf) = 0
-        negd[qb] = ok ? a.delta[sidx] : 0.f;
+        const float nd = ok ? a.delta[sidx] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) negd[qb][v] = nd;
 #pragma unroll
         for (int n = 0; n < C::MB; ++n)
 #pragma unroll
@@ -255,7 +260,7 @@ bwd_dq_kernel(const BwdArgs a) {
                     f32x16_t s, dp;
                     const int query = wq0 + qb * 32 + c;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) s[v] = dp[v] = 0.f;
+                    for (int v = 0; v < 16; ++v) s[v] = 0.f;
                     // q k^T and q_b k_b^T: two independent MFMA chains, joined by one FMA per score
                     // that applies the softmax scale in fp32 (:638-641); an additive mask is the
                     // initial value of the bias chain
@@ -283,7 +288,7 @@ bwd_dq_kernel(const BwdArgs a) {
                         for (int v = 0; v < 16; ++v) s[v] *= a.scale;
                     }
 #pragma unroll
-                    for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], dp);
+                    for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], t == 0 ? negd[qb] : dp);
                     const bool edge = (n0 + kb * 32 + 32 > a.Lk) || (a.causal && n0 + kb * 32 + 31 > wq0 + qb * 32);
                     if (edge) {
 #pragma unroll
@@ -296,7 +301,7 @@ bwd_dq_kernel(const BwdArgs a) {
                     for (int v = 0; v < 16; v += 2) {
                         const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[qb]));
                         const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[qb]));
-                        dsp[qb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * (dp[v] + negd[qb]), p1 * (dp[v + 1] + negd[qb]));
+                        dsp[qb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
                     }
                 }
                 // [dQ | dQ_b]^T += [K | K_b]^T dS^T over this block's 32 keys
