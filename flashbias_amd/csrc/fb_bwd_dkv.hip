@@ -25,16 +25,23 @@
 
 namespace fb {
 
-template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_>
+// PART: 0 = dv, dk and dk_bias in one pass; 1 = dv only; 3 / 4 = the lower / upper half of the
+// 32-row blocks of [dk | dk_bias] only.  Head dims above 64 run as three launches (1, 3, 4) with
+// 32-query steps: each pass keeps its accumulators in registers and its LDS stages small enough
+// for two waves per SIMD, which is worth recomputing S.
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, int PART_ = 0>
 struct DkvCfg {
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
+    static constexpr bool DO_DV = PART_ <= 1, DO_DK = PART_ != 1;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dK | dK_b]^T
+    // ... of which this instantiation accumulates [MB0, MB1)
+    static constexpr int MB0 = PART_ == 4 ? MB / 2 : 0, MB1 = PART_ == 1 ? 0 : PART_ == 3 ? MB / 2 : MB;
     static constexpr int KBW = 1; // key blocks per wave
     static constexpr int BN = 32 * KBW * NWAVES;              // keys per workgroup
-    static constexpr int QBLK = 2, BMQ = 32 * QBLK;           // queries per step
+    static constexpr int QBLK = PART_ == 0 ? 2 : 1, BMQ = 32 * QBLK; // queries per step
     // sQ row: [Q | Q_b] of one query, sdO row: dout of one query, both in swizzled 16-byte
     // chunks; each tile is kept once and read row-wise (S, dP) and column-wise (dK, dV)
     static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
@@ -54,7 +61,7 @@ struct DkvCfg {
     static constexpr int CQ = 2 * NKD, CR = 2 * NKR, CO = 2 * NKD;
     static constexpr int TASKS = BMQ * (CQ + CR + CO);
     static constexpr int PT = (TASKS + NTHREADS - 1) / NTHREADS;
-    static constexpr int WAVES_EU = (NK <= 6 && NDV <= 2) ? 2 : 1;
+    static constexpr int WAVES_EU = ((NK <= 6 && NDV <= 2) || PART_ != 0) ? 2 : 1;
 };
 
 template <class C>
@@ -159,7 +166,7 @@ struct DkvDirect {
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *qbase, const uint16_t *qbbase,
                                          const uint16_t *dobase, const float *lse2, const float *negd, int wave_,
                                          int lane_) {
-        static_assert(C::BMQ == 64, "one statistics row per copy instruction");
+        static_assert(C::BMQ <= 64, "one statistics row per copy instruction");
         wave = wave_;
         lane = lane_;
         stat = wave == 0 ? lse2 : wave == 1 ? negd : nullptr;
@@ -179,7 +186,8 @@ struct DkvDirect {
         const uint32_t base = lds_addr_of(stage);
         q.issue(base, m0, Lq);
         d.issue(base + 2 * C::SQ, m0, Lq);
-        if (wave < 2) lds_dma4(stat + min(m0 + lane, Lq - 1), base + 2 * (C::SQ + C::SDO) + wave * (4 * C::BMQ));
+        if (wave < 2 && lane < C::BMQ)
+            lds_dma4(stat + min(m0 + lane, Lq - 1), base + 2 * (C::SQ + C::SDO) + wave * (4 * C::BMQ));
         if constexpr (C::MTILE) {
             if (mtile) m.issue(base + 2 * (C::SQ + C::SDO + 4 * C::BMQ), m0, Lq);
         }
@@ -246,8 +254,8 @@ bwd_dkv_kernel(const BwdArgs a) {
 
     // ---- key-side operands, resident in registers
     u32x4_t kreg[C::KBW][C::NK];  // B operand of S: this lane's key, channels 16t + 8g ..
-    u32x4_t vreg[C::KBW][C::NKD]; // B operand of dP
-    f32x16_t acc_dv[C::KBW][C::NDV], acc_dk[C::KBW][C::MB];
+    u32x4_t vreg[C::KBW][C::DO_DK ? C::NKD : 1]; // B operand of dP
+    f32x16_t acc_dv[C::KBW][C::DO_DV ? C::NDV : 1], acc_dk[C::KBW][C::DO_DK ? C::MB1 - C::MB0 : 1];
 #pragma unroll
     for (int kb = 0; kb < C::KBW; ++kb) {
         const int key = wk0 + kb * 32 + c;
@@ -258,15 +266,17 @@ bwd_dkv_kernel(const BwdArgs a) {
             else if constexpr (C::NKR > 0)
                 kreg[kb][t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, 16 * (t - C::NKD) + 8 * g, a.r);
         }
+        if constexpr (C::DO_DK) {
 #pragma unroll
-        for (int t = 0; t < C::NKD; ++t)
-            vreg[kb][t] = load_chunk<C::VEC>(vbase, a.v.ss, key, a.Lk, 16 * t + 8 * g, a.d);
+            for (int t = 0; t < C::NKD; ++t)
+                vreg[kb][t] = load_chunk<C::VEC>(vbase, a.v.ss, key, a.Lk, 16 * t + 8 * g, a.d);
+        }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
 #pragma unroll
-            for (int n = 0; n < C::NDV; ++n) acc_dv[kb][n][v] = 0.f;
+            for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n) acc_dv[kb][n][v] = 0.f;
 #pragma unroll
-            for (int n = 0; n < C::MB; ++n) acc_dk[kb][n][v] = 0.f;
+            for (int n = 0; n < C::MB1 - C::MB0; ++n) acc_dk[kb][n][v] = 0.f;
         }
     }
 
@@ -356,7 +366,7 @@ bwd_dkv_kernel(const BwdArgs a) {
                 for (int t = 0; t < C::NK; ++t)
                     qa[t] = *reinterpret_cast<const u32x4_t *>(sQ + swz_off<C::ROWCH>(qb * 32 + c, 2 * t + g));
 #pragma unroll
-                for (int t = 0; t < C::NKD; ++t)
+                for (int t = 0; t < (C::DO_DK ? C::NKD : 0); ++t)
                     da[t] = *reinterpret_cast<const u32x4_t *>(sdO + swz_off<C::ROWCHO>(qb * 32 + c, 2 * t + g));
                 u32x4_t pp[C::KBW][2], pds[C::KBW][2]; // P and dS, packed, per 16-query step
 #pragma unroll
@@ -381,7 +391,7 @@ bwd_dkv_kernel(const BwdArgs a) {
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
 #pragma unroll
-                    for (int t = 0; t < C::NKD; ++t) dp = T::mfma(da[t], vreg[kb][t], dp);
+                    for (int t = 0; t < (C::DO_DK ? C::NKD : 0); ++t) dp = T::mfma(da[t], vreg[kb][t], dp);
                     f32x16_t mval; // additive mask of this block, added by the FMA that applies the scale
                     if constexpr (C::MASK) {
                         if (mtile) { // column `key`, rows in C-layout order: four transposing reads
@@ -420,24 +430,25 @@ bwd_dkv_kernel(const BwdArgs a) {
                     for (int v = 0; v < 16; v += 2) {
                         const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[v]));
                         const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[v + 1]));
-                        pp[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0, p1);
-                        pds[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
+                        if constexpr (C::DO_DV) pp[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0, p1);
+                        if constexpr (C::DO_DK) pds[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
                     }
                 }
                 // dV^T += dout^T P ; [dK|dK_b]^T += [Q|Q_b]^T dS  (contraction over this block's queries)
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
 #pragma unroll
-                    for (int n = 0; n < C::NDV; ++n) {
+                    for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n) {
                         const u32x4_t dot = lds_read_a_tr<C::ROWCHO>(sdO, qb * 32 + 16 * t, 32 * n, c, g);
 #pragma unroll
                         for (int kb = 0; kb < C::KBW; ++kb) acc_dv[kb][n] = T::mfma(dot, pp[kb][t], acc_dv[kb][n]);
                     }
 #pragma unroll
-                    for (int n = 0; n < C::MB; ++n) {
+                    for (int n = C::MB0; n < C::MB1; ++n) {
                         const u32x4_t qt = lds_read_a_tr<C::ROWCH>(sQ, qb * 32 + 16 * t, 32 * n, c, g);
 #pragma unroll
-                        for (int kb = 0; kb < C::KBW; ++kb) acc_dk[kb][n] = T::mfma(qt, pds[kb][t], acc_dk[kb][n]);
+                        for (int kb = 0; kb < C::KBW; ++kb)
+                            acc_dk[kb][n - C::MB0] = T::mfma(qt, pds[kb][t], acc_dk[kb][n - C::MB0]);
                     }
                 }
             }
@@ -476,7 +487,7 @@ bwd_dkv_kernel(const BwdArgs a) {
             if constexpr (C::NKR > 0)
                 dkbrow = const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + (int64_t)key * a.dkb.ss;
 #pragma unroll
-            for (int n = 0; n < C::NDV; ++n)
+            for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n)
 #pragma unroll
                 for (int bq = 0; bq < 4; ++bq) {
                     const int ch = 32 * n + 8 * bq + 4 * g;
@@ -492,32 +503,32 @@ bwd_dkv_kernel(const BwdArgs a) {
                     }
                 }
 #pragma unroll
-            for (int n = 0; n < C::MB; ++n)
+            for (int n = C::MB0; n < C::MB1; ++n)
 #pragma unroll
                 for (int bq = 0; bq < 4; ++bq) {
                     const int ch = 32 * n + 8 * bq + 4 * g;
                     if (ch < 16 * C::NKD) {
                         if (C::VEC && a.dk.vec_ok && ch + 4 <= a.d) {
                             u32x2_t pk;
-                            pk[0] = T::pack2(acc_dk[kb][n][4 * bq] * a.scale, acc_dk[kb][n][4 * bq + 1] * a.scale);
-                            pk[1] = T::pack2(acc_dk[kb][n][4 * bq + 2] * a.scale, acc_dk[kb][n][4 * bq + 3] * a.scale);
+                            pk[0] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq] * a.scale, acc_dk[kb][n - C::MB0][4 * bq + 1] * a.scale);
+                            pk[1] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq + 2] * a.scale, acc_dk[kb][n - C::MB0][4 * bq + 3] * a.scale);
                             *reinterpret_cast<u32x2_t *>(dkrow + ch) = pk;
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                if (ch + e < a.d) dkrow[ch + e] = T::from_float(acc_dk[kb][n][4 * bq + e] * a.scale);
+                                if (ch + e < a.d) dkrow[ch + e] = T::from_float(acc_dk[kb][n - C::MB0][4 * bq + e] * a.scale);
                         }
                     } else if constexpr (C::NKR > 0) {
                         const int cr = ch - 16 * C::NKD;
                         if (C::VEC && a.dkb.vec_ok && cr + 4 <= a.r) {
                             u32x2_t pk;
-                            pk[0] = T::pack2(acc_dk[kb][n][4 * bq], acc_dk[kb][n][4 * bq + 1]);
-                            pk[1] = T::pack2(acc_dk[kb][n][4 * bq + 2], acc_dk[kb][n][4 * bq + 3]);
+                            pk[0] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq], acc_dk[kb][n - C::MB0][4 * bq + 1]);
+                            pk[1] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq + 2], acc_dk[kb][n - C::MB0][4 * bq + 3]);
                             *reinterpret_cast<u32x2_t *>(dkbrow + cr) = pk;
                         } else {
 #pragma unroll
                             for (int e = 0; e < 4; ++e)
-                                if (cr + e < a.r) dkbrow[cr + e] = T::from_float(acc_dk[kb][n][4 * bq + e]);
+                                if (cr + e < a.r) dkbrow[cr + e] = T::from_float(acc_dk[kb][n - C::MB0][4 * bq + e]);
                         }
                     }
                 }
@@ -525,9 +536,9 @@ bwd_dkv_kernel(const BwdArgs a) {
     }
 }
 
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
-static hipError_t launch_dkv_vec(const BwdArgs &a0, hipStream_t stream) {
-    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK> C;
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART>
+static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
+    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK, PART> C;
     BwdArgs a = a0;
     a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
     auto kern = bwd_dkv_kernel<T, C>;
@@ -539,6 +550,20 @@ static hipError_t launch_dkv_vec(const BwdArgs &a0, hipStream_t stream) {
     const int total = a.ntiles_n * a.B * a.H;
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
+}
+
+// One pass, or (head dims above 64, aligned tensors) a dv pass followed by two dk passes.
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+static hipError_t launch_dkv_vec(const BwdArgs &a, hipStream_t stream) {
+    if constexpr (NKD > 4 && VEC) {
+        hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 1>(a, stream);
+        if (e != hipSuccess) return e;
+        e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 3>(a, stream);
+        if (e != hipSuccess) return e;
+        return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 4>(a, stream);
+    } else {
+        return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 0>(a, stream);
+    }
 }
 
 template <class T, int NKD, int NKR, int NDV>
