@@ -152,11 +152,11 @@ __device__ __forceinline__ void dkv_store_step(const DkvStage<C> &st, const BwdA
 // tiles of a step plus its statistics rows, copied straight into an LDS stage.
 template <class C>
 struct DkvDirect {
-    TileDma<C::BMQ, C::ROWCH, C::NWAVES> q;
-    TileDma<C::BMQ, C::ROWCHO, C::NWAVES> d;
-    TileDma<C::BMQ, C::MROWCH, C::NWAVES> m; // mask tile (masked instantiations, 16-bit matrix masks)
+    TileDma<C::BMQ, C::ROWCH, C::NWAVES, (C::NKR > 0)> q;
+    TileDma<C::BMQ, C::ROWCHO, C::NWAVES, false> d;
+    TileDma<C::BMQ, C::MROWCH, C::NWAVES, false> m; // mask tile (masked instantiations, 16-bit matrix masks)
     bool mtile;
-    static constexpr int N = decltype(q)::NI + decltype(d)::NI;
+    static constexpr int N = decltype(q)::NINST + decltype(d)::NINST;
     // waves 0 and 1 also fetch the step's lse * log2(e) and -delta rows (BMQ = 64 floats: one
     // 4-byte copy per lane)
     static constexpr int NS = 1;
@@ -165,31 +165,31 @@ struct DkvDirect {
 
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *qbase, const uint16_t *qbbase,
                                          const uint16_t *dobase, const float *lse2, const float *negd, int wave_,
-                                         int lane_) {
+                                         int lane_, int m0) {
         static_assert(C::BMQ <= 64, "one statistics row per copy instruction");
         wave = wave_;
         lane = lane_;
         stat = wave == 0 ? lse2 : wave == 1 ? negd : nullptr;
-        q.init(qbase, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? qbbase : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane);
-        d.init(dobase, a.dout.ss, a.d, C::ROWCHO, nullptr, 0, 0, wave, lane);
+        q.init(qbase, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? qbbase : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane, m0);
+        d.init(dobase, a.dout.ss, a.d, C::ROWCHO, nullptr, 0, 0, wave, lane, m0);
         mtile = false;
     }
 
     // The workgroup's columns [n0, n0 + BN) of the (batch, head) mask matrix, 16-bit elements.
-    __device__ __forceinline__ void init_mask(const BwdArgs &a, const uint8_t *mbase, int n0) {
+    __device__ __forceinline__ void init_mask(const BwdArgs &a, const uint8_t *mbase, int n0, int m0) {
         mtile = true;
         const int ncols = a.Lk - n0 < C::BN ? a.Lk - n0 : C::BN;
-        m.init(reinterpret_cast<const uint16_t *>(mbase) + n0, a.mask.sm, ncols, C::MROWCH, nullptr, 0, 0, wave, lane);
+        m.init(reinterpret_cast<const uint16_t *>(mbase) + n0, a.mask.sm, ncols, C::MROWCH, nullptr, 0, 0, wave, lane, m0);
     }
 
-    __device__ __forceinline__ void issue(uint16_t *stage, int m0, int Lq) const {
+    __device__ __forceinline__ void issue(const BwdArgs &a, uint16_t *stage, int m0, int Lq) {
         const uint32_t base = lds_addr_of(stage);
-        q.issue(base, m0, Lq);
-        d.issue(base + 2 * C::SQ, m0, Lq);
+        q.issue(base, m0, Lq, a.q.ss, C::NKR > 0 ? a.qb.ss : 0, 2 * C::NKD);
+        d.issue(base + 2 * C::SQ, m0, Lq, a.dout.ss, 0, C::ROWCHO);
         if (wave < 2 && lane < C::BMQ)
             lds_dma4(stat + min(m0 + lane, Lq - 1), base + 2 * (C::SQ + C::SDO) + wave * (4 * C::BMQ));
         if constexpr (C::MTILE) {
-            if (mtile) m.issue(base + 2 * (C::SQ + C::SDO + 4 * C::BMQ), m0, Lq);
+            if (mtile) m.issue(base + 2 * (C::SQ + C::SDO + 4 * C::BMQ), m0, Lq, a.mask.sm, 0, C::MROWCH);
         }
     }
 
@@ -296,16 +296,16 @@ bwd_dkv_kernel(const BwdArgs a) {
     DkvDirect<C> direct;
     DkvStage<C> st;
     if constexpr (C::VEC) {
-        direct.init(a, qbase, qbbase, dobase, lse2, negd, wave, lane);
+        direct.init(a, qbase, qbbase, dobase, lse2, negd, wave, lane, step0 * C::BMQ);
         if constexpr (C::MTILE) {
             // a 16-bit matrix mask whose rows allow 16-byte copies goes through the LDS stages
-            if (a.mask.type == 2 && a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 &&
+            if (a.mask.type == 2 && a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 && a.mask.sm < (1 << 24) &&
                 reinterpret_cast<uintptr_t>(mbase) % 16 == 0)
-                direct.init_mask(a, mbase, n0);
+                direct.init_mask(a, mbase, n0, step0 * C::BMQ);
         }
 #pragma unroll
         for (int k = 0; k < AHEAD; ++k)
-            if (step0 + k < nsteps) direct.issue(stage0 + k * C::STAGE_ELEMS, (step0 + k) * C::BMQ, a.Lq);
+            if (step0 + k < nsteps) direct.issue(a, stage0 + k * C::STAGE_ELEMS, (step0 + k) * C::BMQ, a.Lq);
         // the first step's tiles must have landed; the second step's may still be in flight
         if (AHEAD == 2 && step0 + 1 < nsteps)
             direct.template wait_older<true>();
@@ -345,7 +345,7 @@ bwd_dkv_kernel(const BwdArgs a) {
         if constexpr (C::VEC) {
             if (step + AHEAD < nsteps) {
                 const int tgt = (cur + AHEAD) % C::NSTAGE; // the stage that step - 1 has left
-                direct.issue(stage0 + tgt * C::STAGE_ELEMS, m0 + AHEAD * C::BMQ, a.Lq);
+                direct.issue(a, stage0 + tgt * C::STAGE_ELEMS, m0 + AHEAD * C::BMQ, a.Lq);
             }
             direct.fix_ragged(stage0 + cur * C::STAGE_ELEMS, m0, a.Lq, tid);
         } else if (more) {
@@ -568,8 +568,8 @@ static hipError_t launch_dkv_vec(const BwdArgs &a, hipStream_t stream) {
 
 template <class T, int NKD, int NKR, int NDV>
 static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
-    // the direct loader keeps row strides in 32 bits
-    const int64_t lim = (int64_t)1 << 31;
+    // the direct loader keeps the byte distance between two steps' rows in 32 bits
+    const int64_t lim = (int64_t)1 << 24;
     const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
                      (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0)) && a.q.ss < lim && a.dout.ss < lim &&
                      (a.r == 0 || a.qb.ss < lim);

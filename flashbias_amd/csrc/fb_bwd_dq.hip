@@ -116,20 +116,20 @@ struct DqLoader {
 // a key tile, copied straight into an LDS stage.
 template <class C>
 struct DqDirect {
-    TileDma<C::BN, C::ROWCH, C::NWAVES> k;
-    TileDma<C::BN, C::ROWCHV, C::NWAVES> v;
-    static constexpr int N = decltype(k)::NI + decltype(v)::NI;
+    TileDma<C::BN, C::ROWCH, C::NWAVES, (C::NKR > 0)> k;
+    TileDma<C::BN, C::ROWCHV, C::NWAVES, false> v;
+    static constexpr int N = decltype(k)::NINST + decltype(v)::NINST;
 
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *kbase, const uint16_t *kbbase,
                                          const uint16_t *vbase, int wave, int lane) {
-        k.init(kbase, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? kbbase : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane);
-        v.init(vbase, a.v.ss, a.d, C::ROWCHV, nullptr, 0, 0, wave, lane);
+        k.init(kbase, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? kbbase : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane, 0);
+        v.init(vbase, a.v.ss, a.d, C::ROWCHV, nullptr, 0, 0, wave, lane, 0);
     }
 
-    __device__ __forceinline__ void issue(uint16_t *stage, int n0, int Lk) const {
+    __device__ __forceinline__ void issue(const BwdArgs &a, uint16_t *stage, int n0, int Lk) {
         const uint32_t base = lds_addr_of(stage);
-        k.issue(base, n0, Lk);
-        v.issue(base + 2 * C::SK, n0, Lk);
+        k.issue(base, n0, Lk, a.k.ss, C::NKR > 0 ? a.kb.ss : 0, 2 * C::NKD);
+        v.issue(base + 2 * C::SK, n0, Lk, a.v.ss, 0, C::ROWCHV);
     }
 };
 
@@ -219,7 +219,7 @@ bwd_dq_kernel(const BwdArgs a) {
         direct.init(a, kbase, kbbase, vbase, wave, lane);
 #pragma unroll
         for (int k = 0; k < AHEAD; ++k)
-            if (k < ntiles_k) direct.issue(stage0 + k * C::STAGE, k * C::BN, a.Lk);
+            if (k < ntiles_k) direct.issue(a, stage0 + k * C::STAGE, k * C::BN, a.Lk);
         if (1 < ntiles_k)
             wait_vmcnt<DqDirect<C>::N>(); // the first tile has landed, the second may be in flight
         else
@@ -237,7 +237,7 @@ bwd_dq_kernel(const BwdArgs a) {
         const int nxt = cur == C::NSTAGE - 1 ? 0 : cur + 1;
         if constexpr (C::VEC) {
             if (it + AHEAD < ntiles_k)
-                direct.issue(stage0 + ((cur + AHEAD) % C::NSTAGE) * C::STAGE, n0 + AHEAD * C::BN, a.Lk);
+                direct.issue(a, stage0 + ((cur + AHEAD) % C::NSTAGE) * C::STAGE, n0 + AHEAD * C::BN, a.Lk);
         } else if (more) {
             DqLoader<C>::load(st, a, kbase, kbbase, vbase, n0 + C::BN, tid);
         }
@@ -389,8 +389,11 @@ static hipError_t launch_dq_vec(const BwdArgs &a0, hipStream_t stream) {
 
 template <class T, int NKD, int NKR>
 static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
+    // the direct loader keeps the byte distance between two tiles' rows in 32 bits
+    const int64_t lim = (int64_t)1 << 24;
     const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
-                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0)) && a.k.ss < lim && a.v.ss < lim &&
+                     (a.r == 0 || a.kb.ss < lim);
     if (a.mask.type)
         return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
     return vec ? launch_dq_vec<T, NKD, NKR, true, false>(a, stream) : launch_dq_vec<T, NKD, NKR, false, false>(a, stream);

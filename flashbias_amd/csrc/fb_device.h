@@ -173,6 +173,16 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
 __device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(g) : "memory");
 }
+// 16 bytes per lane from base + off (base wave-uniform, off a 32-bit byte offset per lane), with
+// only the given lanes switched on.  All lanes of the wave must be active at the call.
+__device__ __forceinline__ void lds_dma16_lanes(uint32_t off, const void *base, uint32_t lds, uint64_t lanes) {
+    uint64_t saved;
+    asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
+                 : "=&s"(saved)
+                 : "v"(off), "s"(base), "s"(lds), "s"(lanes)
+                 : "memory");
+}
 __device__ __forceinline__ void lds_dma4(const void *g, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds), "v"(g) : "memory");
 }
@@ -184,27 +194,37 @@ __device__ __forceinline__ void wait_vmcnt() { // at most N vector memory loads 
 __device__ __forceinline__ void barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // One wave's share of the direct copies that fill a swizzled LDS tile of ROWS rows x ROWCH
-// 16-byte chunks from one or two row-major tensors: chunks [0, split) of a tile row come from
-// tensor A (channels 8 * chunk ..), chunks from `split` on from tensor B.  One copy
-// instruction fills 64 consecutive chunk positions of the tile and each lane fetches the global
-// chunk that the swizzle puts at its position.  Lanes whose position is channel padding stay
-// switched off (those chunks keep the zeros of the initial clear); rows past the end of the
-// tensor re-read its last row.  The NWAVES waves of the workgroup issue equal shares.  Every copy
-// instruction has active lanes (each tile row starts with a valid chunk, ncols_a >= 8), so a
-// wave always issues exactly NI of them per tile: the kernels' vmcnt waits count on that.
-template <int ROWS, int ROWCH, int NWAVES>
+// 16-byte chunks from one or (HASB) two row-major tensors: chunks [0, split) of a tile row come
+// from tensor A (channels 8 * chunk ..), chunks from `split` on from tensor B.  One copy
+// instruction fills 64 consecutive chunk positions of the tile, each lane fetching the global
+// chunk that the swizzle puts at its position; with two tensors there is one instruction per
+// tensor and group of 64 positions, each with only that tensor's lanes switched on.  Lanes whose
+// position is channel padding are never switched on (those chunks keep the zeros of the initial
+// clear); rows past the end of the tensor re-read its last row.
+//
+// Addressing: the tensor's running tile pointer lives in scalar registers and each lane adds a
+// 32-bit offset that does not change from tile to tile, so a copy costs no vector arithmetic.
+// Tiles must be copied in sequence (rows r0, r0 + ROWS, ...).  The NWAVES waves of the workgroup
+// issue equal shares, and every instruction has lanes switched on (each tile row starts with a
+// valid chunk of every tensor), so a wave always issues exactly NINST of them per tile: the
+// kernels' vmcnt waits count on that.
+template <int ROWS, int ROWCH, int NWAVES, bool HASB>
 struct TileDma {
-    static constexpr int NI = ROWS * ROWCH / 64 / NWAVES; // copy instructions per wave
+    static constexpr int NI = ROWS * ROWCH / 64 / NWAVES; // groups of 64 chunk positions per wave
+    static constexpr int NINST = NI * (HASB ? 2 : 1);     // copy instructions per wave and tile
     static_assert(NI * 64 * NWAVES == ROWS * ROWCH, "tile must split evenly over the waves");
-    const uint16_t *src[NI]; // tensor base + channel offset of this lane's chunk
-    uint32_t ld[NI];         // row stride of that tensor (elements)
-    int row[NI];             // tile row this lane fetches
-    bool ok[NI];
-    int wave;
+    uint32_t off[NI];             // this lane's chunk: bytes from its tensor's tile pointer
+    uint64_t lanes_a[NI], lanes_b[NI];
+    const uint8_t *pa, *pb;       // first row of the next tile in A and B (wave-uniform)
+    int wave, lane;
 
+    // r0: first row of the first tile that issue() will copy.  Row strides below 2^24 elements.
     __device__ __forceinline__ void init(const uint16_t *a, int64_t lda, int ncols_a, int split, const uint16_t *b,
-                                         int64_t ldb, int ncols_b, int wave_, int lane) {
+                                         int64_t ldb, int ncols_b, int wave_, int lane_, int r0) {
         wave = wave_;
+        lane = lane_;
+        pa = reinterpret_cast<const uint8_t *>(a) + (int64_t)r0 * lda * 2;
+        pb = HASB ? reinterpret_cast<const uint8_t *>(b) + (int64_t)r0 * ldb * 2 : nullptr;
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
             const int p = (wave * NI + j) * 64 + lane;
@@ -212,21 +232,35 @@ struct TileDma {
             const int chunk = pos ^ swz_of<ROWCH>(r);
             const bool is_b = chunk >= split;
             const int cc = is_b ? chunk - split : chunk;
-            row[j] = r;
-            ok[j] = is_b ? (b != nullptr && cc * 8 < ncols_b) : (cc * 8 < ncols_a);
-            src[j] = ok[j] ? (is_b ? b : a) + cc * 8 : a;
-            ld[j] = ok[j] ? (uint32_t)(is_b ? ldb : lda) : 0u;
+            lanes_a[j] = __builtin_amdgcn_ballot_w64(!is_b && cc * 8 < ncols_a);
+            lanes_b[j] = HASB ? __builtin_amdgcn_ballot_w64(is_b && cc * 8 < ncols_b) : 0;
+            off[j] = (uint32_t)r * (uint32_t)((is_b ? ldb : lda) * 2) + cc * 16;
         }
     }
 
-    // tile <- tensor rows [r0, r0 + ROWS), clamped to nrows - 1
-    __device__ __forceinline__ void issue(uint32_t lds_tile, int r0, int nrows) const {
+    // Copies the next tile, rows [r0, r0 + ROWS) clamped to nrows - 1, and moves on to the one
+    // after it.  lda / ldb as given to init(); all lanes of the wave must be active.
+    __device__ __forceinline__ void issue(uint32_t lds_tile, int r0, int nrows, int64_t lda, int64_t ldb, int split) {
+        if (r0 + ROWS <= nrows) {
 #pragma unroll
-        for (int j = 0; j < NI; ++j) {
-            const int q = min(r0 + row[j], nrows - 1);
-            const uint16_t *g = src[j] + (uint64_t)q * ld[j];
-            if (ok[j]) lds_dma16(g, lds_tile + (wave * NI + j) * 1024);
+            for (int j = 0; j < NI; ++j) {
+                lds_dma16_lanes(off[j], pa, lds_tile + (wave * NI + j) * 1024, lanes_a[j]);
+                if constexpr (HASB) lds_dma16_lanes(off[j], pb, lds_tile + (wave * NI + j) * 1024, lanes_b[j]);
+            }
+        } else { // the ragged last tile: rows past the end step back to the last row
+#pragma unroll
+            for (int j = 0; j < NI; ++j) {
+                const int p = (wave * NI + j) * 64 + lane;
+                const int r = p / ROWCH, pos = p % ROWCH;
+                const bool is_b = (pos ^ swz_of<ROWCH>(r)) >= split;
+                const int over = max(r0 + r - (nrows - 1), 0);
+                const uint32_t o = off[j] - (uint32_t)over * (uint32_t)((is_b ? ldb : lda) * 2);
+                lds_dma16_lanes(o, pa, lds_tile + (wave * NI + j) * 1024, lanes_a[j]);
+                if constexpr (HASB) lds_dma16_lanes(o, pb, lds_tile + (wave * NI + j) * 1024, lanes_b[j]);
+            }
         }
+        pa += lda * (2 * ROWS);
+        if constexpr (HASB) pb += ldb * (2 * ROWS);
     }
 };
 
