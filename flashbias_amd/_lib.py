@@ -13,8 +13,8 @@ FB_F16, FB_BF16, FB_F32 = 0, 1, 2
 FB_MASK_NONE, FB_MASK_VECTOR, FB_MASK_MATRIX = 0, 1, 2
 
 #: every symbol that include/flashbias.h declares
-EXPORTS = ("fb_version", "fb_last_error", "fb_check", "fb_fwd", "fb_bwd", "fb_bwd_preprocess", "fb_bwd_dkv",
-           "fb_bwd_dq")
+EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_check", "fb_fwd", "fb_bwd",
+           "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq")
 
 
 class FbTensor(ctypes.Structure):
@@ -59,6 +59,8 @@ def load():
             raise ImportError(f"{LIB_PATH} does not export {name}")
     lib.fb_version.restype = ctypes.c_int
     lib.fb_last_error.restype = ctypes.c_char_p
+    lib.fb_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FbParams)]
+    lib.fb_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.fb_check.argtypes = [ctypes.POINTER(FbParams), ctypes.c_int]
     lib.fb_check.restype = ctypes.c_int
     for name in ("fb_fwd", "fb_bwd", "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq"):

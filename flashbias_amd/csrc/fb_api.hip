@@ -159,6 +159,11 @@ int fb_version(void) { return FB_VERSION; }
 
 const char *fb_last_error(void) { return g_err; }
 
+size_t fb_bwd_workspace_bytes(const fb_params *p) {
+    if (!p || p->B <= 0 || p->H <= 0 || p->Lq <= 0) return 0;
+    return (size_t)2 * (size_t)p->B * (size_t)p->H * (size_t)p->Lq * sizeof(float);
+}
+
 int fb_check(const fb_params *p, int pass) {
     g_err[0] = 0;
     if (!p) return fail(FB_ERR_NULL, "params: null pointer");

@@ -119,7 +119,8 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
         dqb_full = torch.empty((p.B, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
         dkb_full = torch.empty((p.B, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
         p.dq_bias, p.dk_bias = _tensor(dqb_full), _tensor(dkb_full)
-    delta = torch.empty((2,) + tuple(lse.shape), device=lse.device, dtype=torch.float32)  # -delta, lse*log2(e)
+    # scratch of the backward: -delta and lse * log2(e), sized by the library
+    delta = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=lse.device, dtype=torch.float32)
     p.delta = delta.data_ptr()
     with torch.cuda.device(q.device):
         _lib.check_status(lib.fb_bwd(p, _stream()))

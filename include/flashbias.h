@@ -92,6 +92,11 @@ const char *fb_last_error(void);
  * pass: 0 = forward, 1 = backward. */
 int fb_check(const fb_params *p, int pass);
 
+/* Bytes of the backward's scratch buffer fb_params.delta for these sizes (2 * B * H * Lq floats;
+ * the reference allocates delta, dq_accum and dq_bias_accum itself, flash_bias_triton.py:1212-1219).
+ * Only B, H and Lq are read; returns 0 for a null pointer or non-positive sizes. */
+size_t fb_bwd_workspace_bytes(const fb_params *p);
+
 /* Replaces _flash_attn_forward + _fwd_kernel (flash_bias_triton.py:1100-1194, :62-355):
  * o = softmax(scale q k^T + q_bias k_bias^T + mask) v and lse. */
 int fb_fwd(const fb_params *p, void *stream);

@@ -28,6 +28,16 @@ def test_library_exports_every_declared_symbol():
     assert lib.fb_version() == 1
 
 
+def test_workspace_size_query():
+    lib = _lib.load()
+    p = _lib.new_params()
+    p.B, p.H, p.Lq = 2, 4, 1000
+    assert lib.fb_bwd_workspace_bytes(p) == 2 * 2 * 4 * 1000 * 4
+    p.Lq = 0
+    assert lib.fb_bwd_workspace_bytes(p) == 0
+    assert lib.fb_bwd_workspace_bytes(None) == 0
+
+
 def _good(pass_=0):
     p = _lib.new_params()
     p.dtype = _lib.FB_BF16
