@@ -471,8 +471,11 @@ static hipError_t launch_fwd_vec(const FwdArgs &a0, hipStream_t stream) {
 
 template <class T, int NKD, int NKR, int NDV>
 static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
+    // the fast loader keeps the element offset of a tile row in 32 bits
+    const int64_t lim = (int64_t)1 << 24;
     const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.o.vec_ok && a.d % 8 == 0 &&
-                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0));
+                     (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0)) && a.k.ss < lim && a.v.ss < lim &&
+                     (a.r == 0 || a.kb.ss < lim);
     if (a.mask.type)
         return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);

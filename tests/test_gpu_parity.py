@@ -131,6 +131,29 @@ def test_noncontiguous_inputs_and_scale(gpu_device):
     _gate(got, ref, torch.bfloat16)
 
 
+@pytest.mark.parametrize("stride", [(1 << 24) - 8, 1 << 24])
+def test_huge_row_strides(gpu_device, stride):
+    """Rows 32 MB apart: just below the limit the tile loaders keep their 32-bit offsets, at the
+    limit the kernels must take the element-wise path (64-bit addresses)."""
+    B, L, H, d, r = 1, 5, 1, 32, 8
+    q, k, v, qb, kb, do = make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=21)
+    ref = oracle(q, k, v, qb, kb, None, False, None, do)
+    dev = gpu_device
+
+    def spread(t):  # the same values in rows `stride` elements apart
+        buf = torch.zeros(L * stride, dtype=t.dtype, device=dev)
+        view = buf.as_strided(t.shape, (L * stride, stride, t.shape[-1], 1))
+        view.copy_(t.to(dev))
+        return view.detach().requires_grad_(True)
+
+    leaves = [spread(t) for t in (q, k, v, qb, kb)]
+    assert leaves[0].stride(1) == stride
+    o = flash_bias_func(*leaves, None, False, None)
+    grads = torch.autograd.grad(o, leaves, spread(do).detach())
+    got = [o.detach().float().cpu()] + [g.float().cpu() for g in grads]
+    _gate(got, ref, torch.bfloat16)
+
+
 def test_lse_and_default_scale(gpu_device):
     from flashbias_amd.interface import _flash_bias_forward
     q, k, v, qb, kb, do = make_inputs(2, 300, 260, 2, 64, 8, torch.bfloat16, seed=3)
