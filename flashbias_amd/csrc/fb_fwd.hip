@@ -58,7 +58,10 @@ struct FwdCfg {
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int KB_PT = (KB_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
-    static constexpr int WAVES_EU = QB == 2 ? 2 : (NK <= 4 && NDV <= 2) ? 3 : 2;
+    // registers: three waves per SIMD for the small configurations, one (512 registers) where the
+    // mask values or an unaligned head dim of 128 would spill at 256, else two
+    static constexpr bool BIG = (MASK_ && (NDV_ >= 2 || NKD_ + NKR_ >= 5)) || (!VEC_ && NDV_ == 4);
+    static constexpr int WAVES_EU = QB == 2 ? 2 : BIG ? 1 : (NK <= 4 && NDV <= 2) ? 3 : 2;
     // LDS fragments requested ahead of their use: all key steps of a group when they are few,
     // and the V^T fragments of a group when the head dimension is one MFMA block
     static constexpr int KPRE = NK <= 4 ? NK : 0;
@@ -204,7 +207,7 @@ struct FwdLoader {
 };
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, C::WAVES_EU))) void fwd_kernel(
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU == 1 ? 1 : 2, C::WAVES_EU))) void fwd_kernel(
     const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *sKbuf = reinterpret_cast<uint16_t *>(smem);
