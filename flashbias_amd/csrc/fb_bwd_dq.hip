@@ -21,14 +21,15 @@
 
 namespace fb {
 
-template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_>
+// QB2_: allow two query blocks per wave (the launcher turns it off for small grids).
+template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_, bool QB2_ = true>
 struct DqCfg {
     static constexpr int NKD = NKD_, NKR = NKR_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dQ | dQ_b]^T
-    static constexpr int QBLK = (NK <= 3 && !MASK_) ? 2 : 1; // the mask values need the registers of the second block
+    static constexpr int QBLK = (QB2_ && NK <= 3 && !MASK_) ? 2 : 1; // the mask values need the registers of the second block
     static constexpr int BM = NWAVES * QBLK * 32;
     static constexpr int KBLK = 2, BN = 32 * KBLK;
     // sK row: [K | K_b] of one key in ROWCH swizzled 16-byte chunks; the one copy is read
@@ -134,7 +135,7 @@ struct DqDirect {
 };
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU))) void
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::QBLK == 1 && C::NK <= 3 ? 1 : 0)))) void
 bwd_dq_kernel(const BwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
@@ -371,9 +372,9 @@ bwd_dq_kernel(const BwdArgs a) {
     }
 }
 
-template <class T, int NKD, int NKR, bool VEC, bool MASK>
-static hipError_t launch_dq_vec(const BwdArgs &a0, hipStream_t stream) {
-    typedef DqCfg<T, NKD, NKR, VEC, MASK> C;
+template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2>
+static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
+    typedef DqCfg<T, NKD, NKR, VEC, MASK, QB2> C;
     BwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = bwd_dq_kernel<T, C>;
@@ -385,6 +386,18 @@ static hipError_t launch_dq_vec(const BwdArgs &a0, hipStream_t stream) {
     const int total = a.ntiles_m * a.B * a.H;
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
+}
+
+// 256-query workgroups (two blocks per wave) once every compute unit has two of them (three under
+// a causal mask), 128-query workgroups below that: as in the forward launcher.
+template <class T, int NKD, int NKR, bool VEC, bool MASK>
+static hipError_t launch_dq_vec(const BwdArgs &a, hipStream_t stream) {
+    if constexpr (DqCfg<T, NKD, NKR, VEC, MASK, true>::QBLK == 2) {
+        const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
+        if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus())
+            return launch_dq_qb<T, NKD, NKR, VEC, MASK, false>(a, stream);
+    }
+    return launch_dq_qb<T, NKD, NKR, VEC, MASK, true>(a, stream);
 }
 
 template <class T, int NKD, int NKR>

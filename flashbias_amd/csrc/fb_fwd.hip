@@ -29,14 +29,15 @@
 namespace fb {
 
 // VEC: every streamed tensor is 16-byte aligned (base and strides) and d, r are multiples of 8.
-template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_>
+// QB2_: allow two query blocks per wave (the launcher turns it off for small grids).
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, bool QB2_ = true>
 struct FwdCfg {
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     // query blocks (of 32) per wave: two where the registers allow, so that every key / value
     // fragment read from LDS feeds two blocks and two waves per SIMD carry four softmax streams
-    static constexpr int QB = (NKD_ + NKR_ <= 3 && NDV_ == 1 && VEC_ && !MASK_) ? 2 : 1;
+    static constexpr int QB = (QB2_ && NKD_ + NKR_ <= 3 && NDV_ == 1 && VEC_ && !MASK_) ? 2 : 1;
     static constexpr int BM = NWAVES * 32 * QB;
     static constexpr int NK = NKD + NKR;
     // A wave computes KBLK * 32 keys at a time; an LDS tile (one barrier) holds SUBS such groups.
@@ -456,9 +457,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
     }
 }
 
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
-static hipError_t launch_fwd_vec(const FwdArgs &a0, hipStream_t stream) {
-    typedef FwdCfg<T, NKD, NKR, NDV, VEC, MASK> C;
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool QB2>
+static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
+    typedef FwdCfg<T, NKD, NKR, NDV, VEC, MASK, QB2> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_kernel<T, C>;
@@ -470,6 +471,20 @@ static hipError_t launch_fwd_vec(const FwdArgs &a0, hipStream_t stream) {
     const int total = a.ntiles_m * a.B * a.H;
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
+}
+
+// Two query blocks per wave (256 queries per workgroup) pay once every compute unit has two such
+// workgroups (three under a causal mask, whose tiles differ in length); below that, 128-query
+// workgroups at three waves per SIMD fill the chip better (measured: 35 % faster at a quarter
+// of that grid, 10 % slower at twice it).
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+static hipError_t launch_fwd_vec(const FwdArgs &a, hipStream_t stream) {
+    if constexpr (FwdCfg<T, NKD, NKR, NDV, VEC, MASK, true>::QB == 2) {
+        const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
+        if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus())
+            return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, false>(a, stream);
+    }
+    return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, true>(a, stream);
 }
 
 template <class T, int NKD, int NKR, int NDV>

@@ -36,6 +36,20 @@ hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream
 hipError_t launch_bwd_dkv(const BwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream);
 
+// Compute units of the current device (cached per device; 256 on MI355X).  The launchers pick
+// smaller query tiles when the larger ones would leave compute units without a workgroup.
+inline int num_cus() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cached[dev];
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cached[dev] = n; // (idempotent: concurrent first calls store the same value)
+    }
+    return n;
+}
+
 // Padded sizes the dispatchers use: d is covered by 16-wide contraction steps of the
 // QK^T product (NKD of them) and the rank by NKR more; both rounded up to the next
 // instantiated size (1, 2, 4, 8 steps).
