@@ -246,6 +246,17 @@ def test_long_ragged_sequences(gpu_device, Lq, Lk, causal):
     _case(gpu_device, 1, Lq, Lk, 2, 32, 8, torch.bfloat16, causal, seed=12)
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk,r,causal", [(8, 16, 1000, 1000, 8, False), (8, 32, 700, 700, 8, True),
+                                                 (4, 64, 777, 1300, 16, False), (8, 32, 1300, 777, 0, True),
+                                                 (64, 16, 256, 256, 8, False)])
+def test_large_grids_ragged(gpu_device, B, H, Lq, Lk, r, causal):
+    """Grids of at least two (causal: three) 256-query workgroups per compute unit of an MI355X
+    (256 CUs): the launchers then pick the two-query-blocks-per-wave kernels, which the small
+    cases above never reach; ragged last tiles, rectangular and causal shapes."""
+    assert B * H * ((Lq + 255) // 256) >= (3 if causal else 2) * 256
+    _case(gpu_device, B, Lq, Lk, H, 32, r, torch.bfloat16, causal, seed=13)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("offset", [0, 1])
 def test_matrix_mask_alignment(gpu_device, dtype, offset):
