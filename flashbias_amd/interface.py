@@ -37,6 +37,30 @@ def _last_dim_contiguous(x):
     return x if x.stride(-1) == 1 else x.contiguous()
 
 
+# A vector mask on a problem of at least this many (batch, head, query, key) pairs is folded into
+# the factors (below that the extra tensor operations cost more than the kernels gain: measured
+# at B2 H4 d32 r8, 2.09 against 2.96 ms fwd+bwd at L=16384, 0.38 against 0.32 ms at L=4096).
+_FOLD_MIN_PAIRS = 1 << 29
+
+
+def _fold_vector_mask(q, q_bias, k_bias, mask):
+    """An additive (B|1, H|1, 1, Lk) mask is itself a rank-1 bias, 1_i * mask_j: appended to the
+    factors as one more column it rides through the kernels' rank steps (which pad the rank to
+    a multiple of 16 anyway) instead of being loaded by every query tile.  Exact for a mask of
+    the input dtype: the products 1 * mask_j are summed in fp32 like every other bias term, and
+    -inf entries stay -inf.  Returns (q_bias', k_bias'); the gradients of the added columns
+    are dropped by the caller."""
+    batch, seqlen_q, nheads, _ = q.shape
+    seqlen_k = mask.shape[-1]
+    col = mask.permute(0, 3, 1, 2)  # (B|1, Lk, H|1, 1)
+    if q_bias is None:
+        return q.new_ones((1, seqlen_q, 1, 1)), col
+    kb, hb = max(k_bias.shape[0], col.shape[0]), max(k_bias.shape[2], col.shape[2])
+    k_new = torch.cat([k_bias.expand(kb, seqlen_k, hb, -1), col.expand(kb, seqlen_k, hb, 1)], dim=-1)
+    q_new = torch.cat([q_bias, q_bias.new_ones(q_bias.shape[:-1] + (1,))], dim=-1)
+    return q_new, k_new
+
+
 def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
     """Argument checks of _flash_attn_forward (flash_bias_triton.py:1100-1143) and the
     parameter block shared by forward and backward.  Returns (params, keepalive)."""
@@ -55,6 +79,11 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
     p.scale = softmax_scale or 1.0 / math.sqrt(d)
     p.q, p.k, p.v = _tensor(q), _tensor(k), _tensor(v)
     keep = []
+    if (mask is not None and mask.dim() == 4 and mask.shape[2] == 1 and mask.shape[3] == seqlen_k
+            and mask.dtype == q.dtype and mask.is_cuda
+            and batch * nheads * seqlen_q * seqlen_k >= _FOLD_MIN_PAIRS):
+        q_bias, k_bias = _fold_vector_mask(q, q_bias, k_bias, mask)
+        mask = None
     if q_bias is not None:
         assert k_bias is not None and q_bias.dtype == k_bias.dtype == q.dtype
         assert q_bias.is_cuda and k_bias.is_cuda
@@ -66,6 +95,8 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
             pad = (0, 8 - rank % 8)
             q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
             rank = q_bias.shape[-1]
+        # (padding a permuted view keeps its permuted layout)
+        q_bias, k_bias = _last_dim_contiguous(q_bias), _last_dim_contiguous(k_bias)
         # stride-0 broadcast over batch / heads (:1135-1136)
         qbe = q_bias.expand(batch, seqlen_q, nheads, rank)
         kbe = k_bias.expand(batch, seqlen_k, nheads, rank)
@@ -115,7 +146,7 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     p.o, p.lse, p.dout = _tensor(o), lse.data_ptr(), _tensor(do)
     p.dq, p.dk, p.dv = _tensor(dq), _tensor(dk), _tensor(dv)
     dqb_full = dkb_full = None
-    if q_bias is not None:
+    if p.r:  # (also when only a folded vector mask makes up the factors)
         dqb_full = torch.empty((p.B, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
         dkb_full = torch.empty((p.B, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
         p.dq_bias, p.dk_bias = _tensor(dqb_full), _tensor(dkb_full)

@@ -108,6 +108,29 @@ def test_additive_mask(gpu_device, kind, causal):
     _case(gpu_device, B, Lq, Lk, H, 32, 8, torch.bfloat16, causal, mask=mask)
 
 
+@pytest.mark.parametrize("r,bmask,hmask,bk", [(8, True, False, (False, False)), (16, False, True, (True, False)),
+                                              (0, True, True, (False, False)), (8, False, False, (True, True))])
+def test_vector_mask_folded_into_factors(gpu_device, monkeypatch, r, bmask, hmask, bk):
+    """On large problems the wrapper passes a vector mask of the input dtype to the kernels as
+    one more factor column (forced here at a small size); key-padding style -inf entries, all
+    broadcast combinations of mask and key factor, and no factors at all."""
+    from flashbias_amd import interface
+    monkeypatch.setattr(interface, "_FOLD_MIN_PAIRS", 0)
+    B, Lq, Lk, H = 2, 300, 520, 4
+    q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, 32, r, torch.bfloat16, seed=31, bk=bk)
+    g = torch.Generator().manual_seed(32)
+    mask = torch.randn(B if bmask else 1, H if hmask else 1, 1, Lk, generator=g).bfloat16()
+    mask[..., Lk - 100:] = float("-inf")
+    mask[0, 0, 0, 5] = float("-inf")
+    ref = oracle(q, k, v, qb, kb, mask, False, None, do)
+    got = run_gpu(flash_bias_func, q, k, v, qb, kb, mask, False, None, do, gpu_device)
+    _gate(got, ref, torch.bfloat16)
+    # the same call through the kernels' own mask path
+    monkeypatch.setattr(interface, "_FOLD_MIN_PAIRS", 1 << 62)
+    got2 = run_gpu(flash_bias_func, q, k, v, qb, kb, mask, False, None, do, gpu_device)
+    _gate(got2, ref, torch.bfloat16)
+
+
 def test_noncontiguous_inputs_and_scale(gpu_device):
     """q, k, v as strided views of a packed qkv projection, as the application modules create
     them; non-default softmax scale."""
