@@ -37,9 +37,14 @@ struct DqCfg {
     static constexpr int ROWCH = 2 * NK <= 8 ? 8 : 2 * NK <= 16 ? 16 : 32;
     static constexpr int ROWCHV = 2 * NKD <= 8 ? 8 : 16; // sV row: V of one key, same chunk swizzle
     static constexpr int SK = BN * ROWCH * 8, SV = BN * ROWCHV * 8;
-    static constexpr int STAGE = SK + SV;
-    // direct loader: three stages, two tiles ahead; element-wise loader: two stages, one ahead
-    static constexpr int AHEAD = VEC_ ? 2 : 1;
+    // masked, aligned instantiations also stage the tile's BM x BN block of a 16-bit matrix mask
+    static constexpr bool MTILE = VEC_ && MASK_;
+    static constexpr int MROWCH = BN / 8; // chunks per mask-tile row
+    static constexpr int SM = MTILE ? BM * BN : 0;
+    static constexpr int STAGE = SK + SV + SM;
+    // direct loader: three stages, two tiles ahead; with a mask tile (or the element-wise loader)
+    // two stages, one ahead
+    static constexpr int AHEAD = (VEC_ && !MASK_) ? 2 : 1;
     static constexpr int NSTAGE = AHEAD + 1;
     static constexpr int LDS_BYTES = NSTAGE * STAGE * 2;
     // loader: 8-channel chunks of K, K_b and V, one key row each
@@ -119,6 +124,8 @@ template <class C>
 struct DqDirect {
     TileDma<C::BN, C::ROWCH, C::NWAVES, (C::NKR > 0)> k;
     TileDma<C::BN, C::ROWCHV, C::NWAVES, false> v;
+    TileDma<C::BM, C::MROWCH, C::NWAVES, false> m; // mask tile (masked instantiations, 16-bit matrix masks)
+    bool mtile = false;
     static constexpr int N = decltype(k)::NINST + decltype(v)::NINST;
 
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *kbase, const uint16_t *kbbase,
@@ -127,11 +134,24 @@ struct DqDirect {
         v.init(vbase, a.v.ss, a.d, C::ROWCHV, nullptr, 0, 0, wave, lane, 0);
     }
 
+    // Rows [m0, m0 + BM) of the (batch, head) mask matrix, 16-bit elements; the tiles follow each
+    // other along the rows (BN keys at a time).
+    __device__ __forceinline__ void init_mask(const BwdArgs &a, const uint8_t *mbase, int m0, int wave, int lane) {
+        mtile = true;
+        m0_ = m0;
+        m.init(reinterpret_cast<const uint16_t *>(mbase), a.mask.sm, C::BN, C::MROWCH, nullptr, 0, 0, wave, lane, m0);
+    }
+
     __device__ __forceinline__ void issue(const BwdArgs &a, uint16_t *stage, int n0, int Lk) {
         const uint32_t base = lds_addr_of(stage);
         k.issue(base, n0, Lk, a.k.ss, C::NKR > 0 ? a.kb.ss : 0, 2 * C::NKD);
         v.issue(base + 2 * C::SK, n0, Lk, a.v.ss, 0, C::ROWCHV);
+        if constexpr (C::MTILE) { // full tiles only: a ragged last tile takes the element path
+            if (mtile && n0 + C::BN <= Lk)
+                m.issue_step(base + 2 * (C::SK + C::SV), m0_, a.Lq, a.mask.sm, 0, C::MROWCH, 2 * C::BN, 0);
+        }
     }
+    int m0_ = 0; // first query of the workgroup (set by init_mask)
 };
 
 template <class T, class C>
@@ -218,10 +238,16 @@ bwd_dq_kernel(const BwdArgs a) {
     DqStage<C> st;
     if constexpr (C::VEC) {
         direct.init(a, kbase, kbbase, vbase, wave, lane);
+        if constexpr (C::MTILE) {
+            // a 16-bit matrix mask whose rows allow 16-byte copies goes through the LDS stages
+            if (a.mask.type == 2 && a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 &&
+                a.mask.sm < (1 << 24) && reinterpret_cast<uintptr_t>(mbase) % 16 == 0)
+                direct.init_mask(a, mbase, m0, wave, lane);
+        }
 #pragma unroll
         for (int k = 0; k < AHEAD; ++k)
             if (k < ntiles_k) direct.issue(a, stage0 + k * C::STAGE, k * C::BN, a.Lk);
-        if (1 < ntiles_k)
+        if (AHEAD == 2 && 1 < ntiles_k)
             wait_vmcnt<DqDirect<C>::N>(); // the first tile has landed, the second may be in flight
         else
             wait_vmcnt<0>();
@@ -268,10 +294,25 @@ bwd_dq_kernel(const BwdArgs a) {
                     if constexpr (C::NKR > 0 || C::MASK) {
                         f32x16_t sb;
                         if constexpr (C::MASK) {
-                            const uint8_t *mrow =
-                                mbase + (a.mask.type == 2 ? (int64_t)min(query, a.Lq - 1) * a.mask.sm : 0) *
-                                            (a.mask.is_f32 ? 4 : 2);
-                            mask_block_keys<T>(a.mask, mrow, n0 + kb * 32, g, a.Lk, sb);
+                            if (C::MTILE && direct.mtile && n0 + C::BN <= a.Lk) {
+                                // this lane's query row of the staged tile, keys in C-layout order
+                                const uint16_t *sM = sV + C::SV;
+                                const int row = wave * 32 + c;
+#pragma unroll
+                                for (int j = 0; j < 4; ++j) {
+                                    const u32x2_t x = *reinterpret_cast<const u32x2_t *>(
+                                        sM + swz_off<C::MROWCH>(row, 4 * kb + j) + 4 * g);
+                                    sb[4 * j + 0] = T::to_float((uint16_t)(x[0] & 0xffffu));
+                                    sb[4 * j + 1] = T::to_float((uint16_t)(x[0] >> 16));
+                                    sb[4 * j + 2] = T::to_float((uint16_t)(x[1] & 0xffffu));
+                                    sb[4 * j + 3] = T::to_float((uint16_t)(x[1] >> 16));
+                                }
+                            } else {
+                                const uint8_t *mrow =
+                                    mbase + (a.mask.type == 2 ? (int64_t)min(query, a.Lq - 1) * a.mask.sm : 0) *
+                                                (a.mask.is_f32 ? 4 : 2);
+                                mask_block_keys<T>(a.mask, mrow, n0 + kb * 32, g, a.Lk, sb);
+                            }
                         } else {
 #pragma unroll
                             for (int v = 0; v < 16; ++v) sb[v] = 0.f;
@@ -317,7 +358,7 @@ bwd_dq_kernel(const BwdArgs a) {
             }
         }
         if constexpr (C::VEC) {
-            if (it + AHEAD < ntiles_k)
+            if (AHEAD == 2 && it + AHEAD < ntiles_k)
                 wait_vmcnt<DqDirect<C>::N>(); // the next tile has landed, the one after may be in flight
             else
                 wait_vmcnt<0>();

@@ -241,6 +241,13 @@ struct TileDma {
     // Copies the next tile, rows [r0, r0 + ROWS) clamped to nrows - 1, and moves on to the one
     // after it.  lda / ldb as given to init(); all lanes of the wave must be active.
     __device__ __forceinline__ void issue(uint32_t lds_tile, int r0, int nrows, int64_t lda, int64_t ldb, int split) {
+        issue_step(lds_tile, r0, nrows, lda, ldb, split, lda * (2 * ROWS), ldb * (2 * ROWS));
+    }
+
+    // The same with the byte distance to the next tile given by the caller (a sequence of tiles
+    // that runs along the rows of the tensor instead of down its columns).
+    __device__ __forceinline__ void issue_step(uint32_t lds_tile, int r0, int nrows, int64_t lda, int64_t ldb, int split,
+                                               int64_t step_a, int64_t step_b) {
         if (r0 + ROWS <= nrows) {
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
@@ -259,8 +266,8 @@ struct TileDma {
                 if constexpr (HASB) lds_dma16_lanes(o, pb, lds_tile + (wave * NI + j) * 1024, lanes_b[j]);
             }
         }
-        pa += lda * (2 * ROWS);
-        if constexpr (HASB) pb += ldb * (2 * ROWS);
+        pa += step_a;
+        if constexpr (HASB) pb += step_b;
     }
 };
 
