@@ -240,7 +240,7 @@ bwd_dq_kernel(const BwdArgs a) {
         direct.init(a, kbase, kbbase, vbase, wave, lane);
         if constexpr (C::MTILE) {
             // a 16-bit matrix mask whose rows allow 16-byte copies goes through the LDS stages
-            if (a.mask.type == 2 && a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 &&
+            if (a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 && // (a vector mask: row stride 0)
                 a.mask.sm < (1 << 24) && reinterpret_cast<uintptr_t>(mbase) % 16 == 0)
                 direct.init_mask(a, mbase, m0, wave, lane);
         }

@@ -44,13 +44,17 @@ struct FwdCfg {
     static constexpr int KBLK = 2, BSUB = 32 * KBLK;
     // two groups per tile where three workgroups of that size still fit the 160 KB of a CU
     static constexpr int LDS2 = 2 * 2 * (2 * BSUB * (16 * NK + 8) + 32 * NDV_ * (2 * BSUB + 8));
-    static constexpr int SUBS = (NK <= 4 && NDV_ <= 2 && 3 * LDS2 <= 160 * 1024) ? 2 : 1;
+    // (masked, aligned instantiations also stage a BM x BN mask tile: one group per tile)
+    static constexpr bool MTILE = VEC_ && MASK_;
+    static constexpr int SUBS = (!MTILE && NK <= 4 && NDV_ <= 2 && 3 * LDS2 <= 160 * 1024) ? 2 : 1;
     static constexpr int BN = BSUB * SUBS;
     static constexpr int DKP = 16 * NK + 8; // LDS row of [K | K_b], elements (16 B of padding)
     static constexpr int DV = 32 * NDV;
     static constexpr int BNP = BN + 8; // LDS row of V^T
     static constexpr int SK_ELEMS = BN * DKP, SV_ELEMS = DV * BNP;
-    static constexpr int LDS_BYTES = 2 * (SK_ELEMS + SV_ELEMS) * 2;
+    static constexpr int MROWCH = BN / 8;                    // 16-byte chunks per mask-tile row
+    static constexpr int SM_ELEMS = MTILE ? BM * BN : 0;      // 16-bit matrix mask tile, swizzled chunks
+    static constexpr int LDS_BYTES = 2 * (SK_ELEMS + SV_ELEMS + SM_ELEMS) * 2;
     // cooperative loader: 8-channel chunks of K and K_b (one key row each), (4 keys x 4
     // channels) blocks of V.  Consecutive threads take consecutive rows / key quads, which
     // keeps the LDS writes free of bank conflicts.
@@ -213,6 +217,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *sKbuf = reinterpret_cast<uint16_t *>(smem);
     uint16_t *sVbuf = sKbuf + 2 * C::SK_ELEMS;
+    uint16_t *sMbuf = sVbuf + 2 * C::SV_ELEMS;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6); // scalar: branches on it are uniform
@@ -286,21 +291,43 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
         else
             ld.load_safe(stg, a, kbase, kbbase, vbase, n0, tid);
     };
+    // Masked, aligned instantiations: a 16-bit matrix mask whose rows allow 16-byte copies travels
+    // as a BM x BN tile straight into LDS, one tile ahead like K and V (full key tiles only; a
+    // ragged last tile and every other kind of mask take the loads of mask_block_keys).
+    TileDma<C::BM, C::MROWCH, C::NWAVES, false> mdma;
+    bool mtile = false;
+    if constexpr (C::MTILE) {
+        static_assert(C::QB == 1, "one query block per wave in masked instantiations");
+        if (a.mask.vec_ok && !a.mask.is_f32 && a.Lk % 8 == 0 && a.mask.sm % 8 == 0 && // (a vector mask: row stride 0)
+            a.mask.sm < (1 << 24) && reinterpret_cast<uintptr_t>(mbase) % 16 == 0) {
+            mtile = true;
+            mdma.init(reinterpret_cast<const uint16_t *>(mbase), a.mask.sm, C::BN, C::MROWCH, nullptr, 0, 0, wave, lane, m0);
+            if (C::BN <= a.Lk) mdma.issue_step(lds_addr_of(sMbuf), m0, a.Lq, a.mask.sm, 0, C::MROWCH, 2 * C::BN, 0);
+        }
+    }
     FwdStage<C> st;
     load_tile(st, 0);
     ld.store(st, sKbuf, sVbuf);
+    if constexpr (C::MTILE) wait_vmcnt<0>();
     __syncthreads();
 
     for (int it = 0; it < ntiles_k; ++it) {
         const int cur = it & 1;
         const int n0 = it * C::BN;
         const bool more = it + 1 < ntiles_k;
+        if constexpr (C::MTILE) {
+            if (mtile && more && n0 + 2 * C::BN <= a.Lk)
+                mdma.issue_step(lds_addr_of(sMbuf + (cur ^ 1) * C::SM_ELEMS), m0, a.Lq, a.mask.sm, 0, C::MROWCH,
+                                2 * C::BN, 0);
+        }
         if (more) load_tile(st, n0 + C::BN);
 
         const uint16_t *sK = sKbuf + cur * C::SK_ELEMS;
         const uint16_t *sVt = sVbuf + cur * C::SV_ELEMS;
+        int nsubs = C::SUBS;
+        if constexpr (C::MTILE) asm volatile("" : "+s"(nsubs)); // keeps the loop a loop (without it the masked code spills)
 #pragma nounroll
-        for (int sub = 0; sub < C::SUBS; ++sub) {
+        for (int sub = 0; sub < nsubs; ++sub) {
             const int ns = n0 + sub * C::BSUB;
             // the group is hidden from every query of this wave: so are all later ones
             if ((a.causal && ns > wq0 + 32 * C::QB - 1) || wq0 >= a.Lq || ns >= k_end) break;
@@ -337,9 +364,26 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
                 if constexpr (C::MASK) {
                     const uint8_t *mrow = mbase + (a.mask.type == 2 ? (int64_t)min(query, a.Lq - 1) * a.mask.sm : 0) *
                                                       (a.mask.is_f32 ? 4 : 2);
+                    if (C::MTILE && mtile && n0 + C::BN <= a.Lk) {
+                        // this lane's query row of the staged tile, keys in C-layout order
+                        const uint16_t *sM = sMbuf + cur * C::SM_ELEMS;
+                        const int row = wave * 32 + c;
 #pragma unroll
-                    for (int kb = 0; kb < C::KBLK; ++kb)
-                        mask_block_keys<T>(a.mask, mrow, ns + kb * 32, g, a.Lk, mk[kb]);
+                        for (int kb = 0; kb < C::KBLK; ++kb)
+#pragma unroll
+                            for (int j = 0; j < 4; ++j) {
+                                const u32x2_t x = *reinterpret_cast<const u32x2_t *>(
+                                    sM + swz_off<C::MROWCH>(row, 4 * kb + j) + 4 * g);
+                                mk[kb][4 * j + 0] = T::to_float((uint16_t)(x[0] & 0xffffu));
+                                mk[kb][4 * j + 1] = T::to_float((uint16_t)(x[0] >> 16));
+                                mk[kb][4 * j + 2] = T::to_float((uint16_t)(x[1] & 0xffffu));
+                                mk[kb][4 * j + 3] = T::to_float((uint16_t)(x[1] >> 16));
+                            }
+                    } else {
+#pragma unroll
+                        for (int kb = 0; kb < C::KBLK; ++kb)
+                            mask_block_keys<T>(a.mask, mrow, ns + kb * 32, g, a.Lk, mk[kb]);
+                    }
                 }
 #pragma unroll
                 for (int kb = 0; kb < C::KBLK; ++kb) {
@@ -424,6 +468,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
             }
         }
         if (more) ld.store(st, sKbuf + (cur ^ 1) * C::SK_ELEMS, sVbuf + (cur ^ 1) * C::SV_ELEMS);
+        if constexpr (C::MTILE) wait_vmcnt<0>(); // the mask tile copies are not known to the compiler
         __syncthreads();
     }
 
