@@ -42,17 +42,21 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a) {
 // Coalesced variant for 16-byte aligned tensors whose rows are 1, 2, 4, 8 or 16 chunks of 8
 // channels: one thread per chunk (consecutive threads read consecutive 16 bytes of a row), the
 // CH partial sums of a row are added across neighbouring lanes.
-template <class T, int CH>
+// IDX: uint32_t when rows * CH fits (the index arithmetic is a good part of this kernel's work
+// and 64-bit divisions are several times as long), else int64_t.
+template <class T, int CH, class IDX>
 __global__ __launch_bounds__(256) void bwd_preprocess_chunks_kernel(const BwdArgs a) {
     const int64_t rows = (int64_t)a.B * a.H * a.Lq;
-    const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t nthreads = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t cix = gid; cix < rows * CH; cix += nthreads) { // rows * CH is a multiple of CH: whole rows per pass
+    const IDX gid = (IDX)blockIdx.x * blockDim.x + threadIdx.x;
+    const IDX nthreads = (IDX)gridDim.x * blockDim.x;
+    const IDX total = (IDX)(rows * CH);
+    for (IDX cix = gid; cix < total; cix += nthreads) { // rows * CH is a multiple of CH: whole rows per pass
         const int c = (int)(cix % CH);
-        const int64_t r = cix / CH; // rows in memory order (b, i, h): neighbouring heads are adjacent
-        const int h = (int)(r % a.H);
-        const int i = (int)((r / a.H) % a.Lq);
-        const int b = (int)(r / ((int64_t)a.H * a.Lq));
+        const IDX r = cix / CH; // rows in memory order (b, i, h): neighbouring heads are adjacent
+        const IDX ri = r / (IDX)a.H;
+        const int h = (int)(r - ri * (IDX)a.H);
+        const int b = (int)(ri / (IDX)a.Lq);
+        const int i = (int)(ri - (IDX)b * (IDX)a.Lq);
         const uint16_t *orow = a.o.ptr + b * a.o.sb + h * a.o.sh + (int64_t)i * a.o.ss;
         const uint16_t *drow = a.dout.ptr + b * a.dout.sb + h * a.dout.sh + (int64_t)i * a.dout.ss;
         float acc = 0.f;
@@ -86,13 +90,21 @@ static void launch_preprocess_t(const BwdArgs &a, hipStream_t stream) {
         int64_t blocks = (rows * ch + 255) / 256;
         if (blocks > 262144) blocks = 262144; // grid-stride beyond that; 256 * blocks stays a multiple of ch
         const dim3 grid((unsigned)blocks), block(256);
+        // (the grid-stride step must not overflow either: 2^30 leaves room for it)
+        const bool small = rows * ch < ((int64_t)1 << 30);
+#define FB_PRE(CHN)                                                                                          \
+    if (small)                                                                                               \
+        hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, CHN, uint32_t>), grid, block, 0, stream, a);     \
+    else                                                                                                     \
+        hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, CHN, int64_t>), grid, block, 0, stream, a);
         switch (ch) {
-        case 1: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 1>), grid, block, 0, stream, a); break;
-        case 2: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 2>), grid, block, 0, stream, a); break;
-        case 4: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 4>), grid, block, 0, stream, a); break;
-        case 8: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 8>), grid, block, 0, stream, a); break;
-        default: hipLaunchKernelGGL((bwd_preprocess_chunks_kernel<T, 16>), grid, block, 0, stream, a); break;
+        case 1: FB_PRE(1) break;
+        case 2: FB_PRE(2) break;
+        case 4: FB_PRE(4) break;
+        case 8: FB_PRE(8) break;
+        default: FB_PRE(16) break;
         }
+#undef FB_PRE
         return;
     }
     int64_t blocks = (rows + 255) / 256;
