@@ -325,7 +325,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
         const uint16_t *sK = sKbuf + cur * C::SK_ELEMS;
         const uint16_t *sVt = sVbuf + cur * C::SV_ELEMS;
         int nsubs = C::SUBS;
-        if constexpr (C::MTILE) asm volatile("" : "+s"(nsubs)); // keeps the loop a loop (without it the masked code spills)
+        if constexpr (C::MTILE || C::SUBS == 1) asm volatile("" : "+s"(nsubs)); // keeps the loop a loop (without it the masked code spills)
 #pragma nounroll
         for (int sub = 0; sub < nsubs; ++sub) {
             const int ns = n0 + sub * C::BSUB;
