@@ -64,7 +64,7 @@ struct DkvCfg {
     // one wave per SIMD (512 registers) where two would spill: large head dims in one pass, and
     // masked instantiations beyond the smallest (they also hold a step's mask values)
     static constexpr bool BIG = MASK_ && PART_ == 0 && (NDV_ >= 2 || NKD_ + NKR_ >= 5);
-    static constexpr int WAVES_EU = BIG ? 1 : ((NK <= 6 && NDV <= 2) || PART_ != 0) ? 2 : 1;
+    static constexpr int WAVES_EU = BIG ? 1 : ((NK <= 8 && NDV <= 2) || PART_ != 0) ? 2 : 1;
 };
 
 template <class C>

@@ -52,7 +52,7 @@ struct DqCfg {
     static constexpr int K_TASKS = BN * (CD + CR), V_TASKS = BN * CD;
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
-    static constexpr int WAVES_EU = (NK <= 6) ? 2 : 1;
+    static constexpr int WAVES_EU = (NK <= (MASK_ ? 6 : 8)) ? 2 : 1;
 };
 
 template <class C>
