@@ -65,7 +65,8 @@ struct FwdCfg {
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
     // registers: three waves per SIMD for the small configurations, one (512 registers) where the
     // mask values or an unaligned head dim of 128 would spill at 256, else two
-    static constexpr bool BIG = (MASK_ && (NDV_ >= 2 || NKD_ + NKR_ >= 5)) || (!VEC_ && NDV_ == 4);
+    static constexpr bool BIG = (MASK_ && (NDV_ >= 2 || NKD_ + NKR_ >= 5)) || (!VEC_ && NDV_ == 4) ||
+                                2 * LDS_BYTES > 160 * 1024; // (one workgroup per CU anyway)
     static constexpr int WAVES_EU = QB == 2 ? 2 : BIG ? 1 : (NK <= 4 && NDV <= 2) ? 3 : 2;
     // LDS fragments requested ahead of their use: all key steps of a group when they are few,
     // and the V^T fragments of a group when the head dimension is one MFMA block
