@@ -71,6 +71,14 @@ def test_ranks(gpu_device, r):
     _case(gpu_device, 1, 160, 224, 2, 32, r, torch.bfloat16, False)
 
 
+@pytest.mark.parametrize("d,r", [(64, 64), (128, 64), (64, 128), (16, 128), (128, 128), (72, 24)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_large_head_dim_and_rank_together(gpu_device, d, r, causal):
+    """Instantiations with many contraction steps: their register budget, LDS footprint and (head
+    dim 128) three-pass dk/dv differ from the small configurations."""
+    _case(gpu_device, 2, 333, 401, 2, d, r, torch.bfloat16, causal, seed=17)
+
+
 @pytest.mark.parametrize("Lq,Lk", [(1, 1), (1, 257), (75, 117), (117, 75), (129, 64), (64, 129), (255, 255)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_ragged_lengths(gpu_device, Lq, Lk, causal):
