@@ -1,6 +1,8 @@
 """CPU tests of the factor builders and workload generators (closed forms and invariants)."""
 import math
 
+import pytest
+
 import torch
 
 from flashbias_amd import factors, workloads
@@ -82,3 +84,33 @@ def test_flop_formulas():
     assert rect == 2 * (1 + 2 + 3 + 3 + 3) * 8
     rf, rfb = workloads.reference_formula_flops(2, 4, 16384, 32)
     assert abs(rf - 2.770e11) < 1e8 and rfb == 3 * rf
+
+
+@pytest.mark.parametrize("r,bmask,hmask,bk,hk", [(8, True, False, False, False), (5, False, True, True, False),
+                                                 (0, True, True, False, False), (16, False, False, True, True)])
+def test_vector_mask_as_factor_column(r, bmask, hmask, bk, hk):
+    """The wrapper's folding of a vector mask into the factors (1_i * mask_j as one more rank) is
+    an identity of the oracle, -inf entries and all broadcast combinations included."""
+    from _util import make_inputs, oracle
+    from flashbias_amd.interface import _fold_vector_mask
+    B, Lq, Lk, H = 2, 37, 53, 3
+    q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, 16, r, torch.float32, seed=5, bk=(bk, hk))
+    g = torch.Generator().manual_seed(6)
+    mask = torch.randn(B if bmask else 1, H if hmask else 1, 1, Lk, generator=g)
+    mask[..., Lk - 9:] = float("-inf")
+    mask[0, 0, 0, 3] = float("-inf")
+    want = oracle(q, k, v, qb, kb, mask, False, None, do)
+    qn, kn = _fold_vector_mask(q, qb, kb, mask)
+    assert qn.shape[-1] == kn.shape[-1] == r + 1
+    got = oracle(q, k, v, qn, kn, None, False, None, do)
+    names = ("o", "lse", "dq", "dk", "dv")
+    for name, a, b in zip(names, got[:5], want[:5]):
+        assert torch.allclose(a, b, rtol=1e-5, atol=1e-5), name
+    if r:
+        # gradients of the original columns; broadcast dims of the folded key factor are summed
+        dqb, dkb = got[5][..., :r], got[6][..., :r]
+        assert torch.allclose(dqb, want[5], rtol=1e-4, atol=1e-5)
+        red = [i for i in (0, 2) if kb.shape[i] == 1 and dkb.shape[i] != 1]
+        if red:
+            dkb = dkb.sum(dim=red, keepdim=True)
+        assert torch.allclose(dkb, want[6], rtol=1e-4, atol=1e-5)
