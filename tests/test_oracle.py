@@ -256,7 +256,7 @@ def _check_blocked(B, Lq, Lk, H, d, r, causal, mask_kind, bm, bn, seed, bq=False
 
 
 def test_blocked_plumbing_config():
-    """BASELINE config 1: fp32, non-causal, B2 H4 L1024 d32 r8."""
+    """The CPU-runnable configuration of the benchmark: fp32, non-causal, B2 H4 L1024 d32 r8."""
     _check_blocked(2, 1024, 1024, 4, 32, 8, False, None, 128, 128, seed=0)
 
 
