@@ -227,6 +227,10 @@ def report(args):
               ("pairformer 768 r32", lambda: workloads.pairformer(), False),
               ("sweep L=4096 + vector mask", lambda: workloads.masked(4096, "vector"), None),
               ("sweep L=4096 + matrix mask", lambda: workloads.masked(4096, "matrix"), None)]
+    # other head dims and ranks at L=8192, and a causal language-model-like shape
+    cases += [(f"sweep L=8192 d={d} r={r}", lambda d=d, r=r: workloads.sweep(8192, d=d, r=r), None)
+              for d, r in ((64, 8), (64, 32), (64, 64), (128, 8), (128, 64))]
+    cases += [("causal B4 H32 L=4096 d=128 r8", lambda: workloads.sweep(4096, B=4, H=32, d=128, causal=True), None)]
     for name, make, dense in cases:
         w = _to_dev(make(), dev)
         B, Lq, H, d = w["q"].shape
