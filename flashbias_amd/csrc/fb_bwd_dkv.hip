@@ -30,8 +30,15 @@ namespace fb {
 // launches (6, 4) while the accumulators of pass 6 fit 256 registers (ranks up to 32), else as
 // three (1, 3, 4), with 32-query steps: each pass keeps its accumulators in registers and its LDS
 // stages small enough for two waves per SIMD, which is worth recomputing S.
-template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, int PART_ = 0>
+// FOLD_: the scores are scale * (q k^T + q_b (k_b / scale)^T), no multiply per score for the scale
+// (the launcher says when that is exact).
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, int PART_ = 0, bool FOLD_ = false>
 struct DkvCfg {
+    static constexpr bool FOLD = FOLD_;
+    static_assert(!FOLD_ || (VEC_ && !MASK_), "folded scale: direct loader, no additive mask");
+    // folded scale with r <= 8: the Q_b columns 8..15 of a step hold a second copy of q_b, the
+    // partner of the low parts of k_b / scale in the key operand
+    static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8; }
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr bool DO_DV = PART_ <= 1 || PART_ == 6, DO_DK = PART_ != 1;
@@ -174,7 +181,8 @@ struct DkvDirect {
         wave = wave_;
         lane = lane_;
         stat = wave == 0 ? lse2 : wave == 1 ? negd : nullptr;
-        q.init(qbase, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? qbbase : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane, m0);
+        q.init(qbase, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? qbbase : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane, m0,
+               C::low_parts(a));
         d.init(dobase, a.dout.ss, a.d, C::ROWCHO, nullptr, 0, 0, wave, lane, m0);
         mtile = false;
     }
@@ -256,6 +264,8 @@ bwd_dkv_kernel(const BwdArgs a) {
         mbase = reinterpret_cast<const uint8_t *>(a.mask.ptr) +
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
+    const float to_log2 = C::FOLD ? a.scale * kLog2e : kLog2e; // the scores are in units of 1 / scale when folded
+
     // ---- key-side operands, resident in registers
     u32x4_t kreg[C::KBW][C::NK];  // B operand of S: this lane's key, channels 16t + 8g ..
     u32x4_t vreg[C::KBW][C::DO_DK ? C::NKD : 1]; // B operand of dP
@@ -267,8 +277,11 @@ bwd_dkv_kernel(const BwdArgs a) {
         for (int t = 0; t < C::NK; ++t) {
             if (t < C::NKD)
                 kreg[kb][t] = load_chunk<C::VEC>(kbase, a.k.ss, key, a.Lk, 16 * t + 8 * g, a.d);
-            else if constexpr (C::NKR > 0)
-                kreg[kb][t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, 16 * (t - C::NKD) + 8 * g, a.r);
+            else if constexpr (C::NKR > 0) {
+                const bool low = C::low_parts(a) && g == 1;
+                kreg[kb][t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, low ? 0 : 16 * (t - C::NKD) + 8 * g, a.r);
+                if constexpr (C::FOLD) kreg[kb][t] = fold_scale_chunk<T>(kreg[kb][t], 1.f / a.scale, C::low_parts(a), low);
+            }
         }
         if constexpr (C::DO_DK) {
 #pragma unroll
@@ -417,9 +430,11 @@ bwd_dkv_kernel(const BwdArgs a) {
                     }
                     // the softmax scale multiplies the fp32 q k^T accumulator before the bias steps
                     // (one chain keeps this kernel at three waves per SIMD)
+                    if constexpr (!C::FOLD) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mval[v]) : s[v] * a.scale;
+                        for (int v = 0; v < 16; ++v)
+                            s[v] = C::MASK ? __builtin_fmaf(s[v], a.scale, mval[v]) : s[v] * a.scale;
+                    }
 #pragma unroll
                     for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
                     const bool edge = (wk0 + kb * 32 + 32 > a.Lk) || (a.causal && wk0 + kb * 32 + 31 > m0 + qb * 32);
@@ -432,8 +447,8 @@ bwd_dkv_kernel(const BwdArgs a) {
                     }
 #pragma unroll
                     for (int v = 0; v < 16; v += 2) {
-                        const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[v]));
-                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[v + 1]));
+                        const float p0 = fast_exp2(__builtin_fmaf(s[v], to_log2, -lse2[v]));
+                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], to_log2, -lse2[v + 1]));
                         if constexpr (C::DO_DV) pp[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0, p1);
                         if constexpr (C::DO_DK) pds[kb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
                     }
@@ -540,9 +555,9 @@ bwd_dkv_kernel(const BwdArgs a) {
     }
 }
 
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART>
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART, bool FOLD>
 static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
-    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK, PART> C;
+    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK, PART, FOLD> C;
     BwdArgs a = a0;
     a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
     auto kern = bwd_dkv_kernel<T, C>;
@@ -558,21 +573,21 @@ static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
 
 // One pass, or (head dims above 64, aligned tensors) two or three passes that each keep a part
 // of the accumulators.
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_dkv_vec(const BwdArgs &a, hipStream_t stream) {
     if constexpr (NKD > 4 && VEC) {
         if constexpr (NKR <= 2 && !MASK) { // two passes: measured 10-18 % faster than three
-            const hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 6>(a, stream);
+            const hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 6, FOLD>(a, stream);
             if (e != hipSuccess) return e;
         } else {
-            hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 1>(a, stream);
+            hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 1, FOLD>(a, stream);
             if (e != hipSuccess) return e;
-            e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 3>(a, stream);
+            e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 3, FOLD>(a, stream);
             if (e != hipSuccess) return e;
         }
-        return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 4>(a, stream);
+        return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 4, FOLD>(a, stream);
     } else {
-        return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 0>(a, stream);
+        return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 0, FOLD>(a, stream);
     }
 }
 
@@ -586,6 +601,9 @@ static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
     if (a.mask.type)
         return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_dkv_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    if constexpr (NKR <= 2) {
+        if (vec && fold_scale_ok<T>(a.scale, a.r)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
+    }
     return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, false>(a, stream)
                : launch_dkv_vec<T, NKD, NKR, NDV, false, false>(a, stream);
 }

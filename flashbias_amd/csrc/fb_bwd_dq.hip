@@ -22,8 +22,15 @@
 namespace fb {
 
 // QB2_: allow two query blocks per wave (the launcher turns it off for small grids).
-template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_, bool QB2_ = true>
+// FOLD_: the scores are scale * (q k^T + (q_b / scale) k_b^T), one MFMA chain and no FMA per
+// score for the scale (the launcher says when that is exact).
+template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_, bool QB2_ = true, bool FOLD_ = false>
 struct DqCfg {
+    static constexpr bool FOLD = FOLD_;
+    static_assert(!FOLD_ || (VEC_ && !MASK_), "folded scale: direct loader, no additive mask");
+    // folded scale with r <= 8: the K_b columns 8..15 of a tile hold a second copy of k_b, the
+    // partner of the low parts of q_b / scale in the query operand
+    static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8; }
     static constexpr int NKD = NKD_, NKR = NKR_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
@@ -130,7 +137,8 @@ struct DqDirect {
 
     __device__ __forceinline__ void init(const BwdArgs &a, const uint16_t *kbase, const uint16_t *kbbase,
                                          const uint16_t *vbase, int wave, int lane) {
-        k.init(kbase, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? kbbase : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane, 0);
+        k.init(kbase, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? kbbase : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane, 0,
+               C::low_parts(a));
         v.init(vbase, a.v.ss, a.d, C::ROWCHV, nullptr, 0, 0, wave, lane, 0);
     }
 
@@ -205,8 +213,11 @@ bwd_dq_kernel(const BwdArgs a) {
         }
         if constexpr (C::NKR > 0) {
 #pragma unroll
-            for (int t = 0; t < C::NKR; ++t)
-                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * t + 8 * g, a.r);
+            for (int t = 0; t < C::NKR; ++t) {
+                const bool low = C::low_parts(a) && g == 1;
+                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, low ? 0 : 16 * t + 8 * g, a.r);
+                if constexpr (C::FOLD) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, C::low_parts(a), low);
+            }
         }
         const bool ok = query < a.Lq;
         const int64_t sidx = (int64_t)bh * a.Lq + (ok ? query : a.Lq - 1);
@@ -220,6 +231,8 @@ bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[qb][n][v] = 0.f;
     }
+
+    const float to_log2 = C::FOLD ? a.scale * kLog2e : kLog2e; // the scores are in units of 1 / scale when folded
 
     int k_end = a.Lk;
     if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
@@ -320,14 +333,23 @@ bwd_dq_kernel(const BwdArgs a) {
 #pragma unroll
                         for (int t = 0; t < C::NKD; ++t) s = T::mfma(ka[t], qr[qb][t], s);
 #pragma unroll
-                        for (int t = C::NKD; t < C::NK; ++t) sb = T::mfma(ka[t], qbr[qb][t - C::NKD], sb);
+                        for (int t = C::NKD; t < C::NK; ++t) {
+                            if constexpr (C::FOLD)
+                                s = T::mfma(ka[t], qbr[qb][t - C::NKD], s);
+                            else
+                                sb = T::mfma(ka[t], qbr[qb][t - C::NKD], sb);
+                        }
+                        if constexpr (!C::FOLD) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) s[v] = __builtin_fmaf(s[v], a.scale, sb[v]);
+                            for (int v = 0; v < 16; ++v) s[v] = __builtin_fmaf(s[v], a.scale, sb[v]);
+                        }
                     } else {
 #pragma unroll
                         for (int t = 0; t < C::NKD; ++t) s = T::mfma(ka[t], qr[qb][t], s);
+                        if constexpr (!C::FOLD) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) s[v] *= a.scale;
+                            for (int v = 0; v < 16; ++v) s[v] *= a.scale;
+                        }
                     }
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], t == 0 ? negd[qb] : dp);
@@ -341,8 +363,8 @@ bwd_dq_kernel(const BwdArgs a) {
                     }
 #pragma unroll
                     for (int v = 0; v < 16; v += 2) {
-                        const float p0 = fast_exp2(__builtin_fmaf(s[v], kLog2e, -lse2[qb]));
-                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], kLog2e, -lse2[qb]));
+                        const float p0 = fast_exp2(__builtin_fmaf(s[v], to_log2, -lse2[qb]));
+                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], to_log2, -lse2[qb]));
                         dsp[qb][v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
                     }
                 }
@@ -413,9 +435,9 @@ bwd_dq_kernel(const BwdArgs a) {
     }
 }
 
-template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2>
+template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2, bool FOLD>
 static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
-    typedef DqCfg<T, NKD, NKR, VEC, MASK, QB2> C;
+    typedef DqCfg<T, NKD, NKR, VEC, MASK, QB2, FOLD> C;
     BwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = bwd_dq_kernel<T, C>;
@@ -431,14 +453,14 @@ static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
 
 // 256-query workgroups (two blocks per wave) once every compute unit has two of them (three under
 // a causal mask), 128-query workgroups below that: as in the forward launcher.
-template <class T, int NKD, int NKR, bool VEC, bool MASK>
+template <class T, int NKD, int NKR, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_dq_vec(const BwdArgs &a, hipStream_t stream) {
     if constexpr (DqCfg<T, NKD, NKR, VEC, MASK, true>::QBLK == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
         if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus())
-            return launch_dq_qb<T, NKD, NKR, VEC, MASK, false>(a, stream);
+            return launch_dq_qb<T, NKD, NKR, VEC, MASK, false, FOLD>(a, stream);
     }
-    return launch_dq_qb<T, NKD, NKR, VEC, MASK, true>(a, stream);
+    return launch_dq_qb<T, NKD, NKR, VEC, MASK, true, FOLD>(a, stream);
 }
 
 template <class T, int NKD, int NKR>
@@ -450,6 +472,9 @@ static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
                      (a.r == 0 || a.kb.ss < lim);
     if (a.mask.type)
         return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
+    if constexpr (NKR <= 2) {
+        if (vec && fold_scale_ok<T>(a.scale, a.r)) return launch_dq_vec<T, NKD, NKR, true, false, true>(a, stream);
+    }
     return vec ? launch_dq_vec<T, NKD, NKR, true, false>(a, stream) : launch_dq_vec<T, NKD, NKR, false, false>(a, stream);
 }
 

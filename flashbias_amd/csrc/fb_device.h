@@ -44,6 +44,7 @@ struct BF16 {
         return __builtin_bit_cast(uint16_t, (__bf16)x);
     }
     static constexpr uint16_t kOne = 0x3f80;
+    static constexpr bool kWideRange = true; // the exponent range of fp32
 };
 
 struct F16 {
@@ -65,6 +66,7 @@ struct F16 {
         return __builtin_bit_cast(uint16_t, (_Float16)x);
     }
     static constexpr uint16_t kOne = 0x3c00;
+    static constexpr bool kWideRange = false;
 };
 
 // A (batch, seq, heads, channels) tensor as the kernels see it: 16-bit elements, channel
@@ -109,6 +111,41 @@ __device__ __forceinline__ u32x4_t load_chunk(const uint16_t *base, int64_t ld, 
         }
 #pragma unroll
         for (int i = 0; i < 4; ++i) out[i] = e[2 * i] | (e[2 * i + 1] << 16);
+    }
+    return out;
+}
+
+// Kernels that fold the softmax scale into the contraction compute scale * (q k^T + q_b' k_b^T)
+// with q_b' = q_b / scale (or k_b' = k_b / scale), the operand that stays in registers.  This
+// turns eight 16-bit values x into rn(x * inv) or, with `split`, into two parts of x * inv: the
+// high part hi (x * inv truncated to 16 bits) or, for `low`, the remainder rn(x * inv - hi).  A
+// lane that owns otherwise unused (zero-padded) columns of the MFMA step carries the low parts
+// there, against a second copy of the other operand's columns, which leaves a relative error of
+// 2^-16 in the product.  Both parts have the sign of x and the low part of a non-zero value is
+// never zero, so that a product with an infinite entry of the other operand (a key-padding
+// column of -inf) is the same infinity in both halves instead of inf - inf or 0 * inf.
+template <class T>
+__device__ __forceinline__ u32x4_t fold_scale_chunk(u32x4_t x, float inv, bool split, bool low) {
+    u32x4_t out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const float f = T::to_float((uint16_t)(hf ? x[e] >> 16 : x[e] & 0xffffu)) * inv;
+            uint16_t hi = T::from_float(f);
+            if (split) {
+                if (fabsf(T::to_float(hi)) > fabsf(f)) hi -= 1; // one step towards zero (sign-magnitude encoding)
+                if (low) {
+                    const float h = T::to_float(hi);
+                    uint16_t lo = (fabsf(h) == INFINITY) ? (uint16_t)0 : T::from_float(f - h);
+                    if ((lo & 0x7fffu) == 0 && fabsf(h) != INFINITY) lo = T::from_float(h * 0x1p-24f);
+                    hi = lo;
+                }
+            }
+            w |= (uint32_t)hi << (16 * hf);
+        }
+        out[e] = w;
     }
     return out;
 }
@@ -219,8 +256,10 @@ struct TileDma {
     int wave, lane;
 
     // r0: first row of the first tile that issue() will copy.  Row strides below 2^24 elements.
+    // twice_b: chunk 1 of the B part of a row is a second copy of chunk 0 (kernels that fold the
+    // softmax scale pair it with the low-order half of the other operand, see fold_scale_chunk).
     __device__ __forceinline__ void init(const uint16_t *a, int64_t lda, int ncols_a, int split, const uint16_t *b,
-                                         int64_t ldb, int ncols_b, int wave_, int lane_, int r0) {
+                                         int64_t ldb, int ncols_b, int wave_, int lane_, int r0, bool twice_b = false) {
         wave = wave_;
         lane = lane_;
         pa = reinterpret_cast<const uint8_t *>(a) + (int64_t)r0 * lda * 2;
@@ -231,7 +270,7 @@ struct TileDma {
             const int r = p / ROWCH, pos = p % ROWCH;
             const int chunk = pos ^ swz_of<ROWCH>(r);
             const bool is_b = chunk >= split;
-            const int cc = is_b ? chunk - split : chunk;
+            const int cc = is_b ? ((twice_b && chunk - split == 1) ? 0 : chunk - split) : chunk;
             lanes_a[j] = __builtin_amdgcn_ballot_w64(!is_b && cc * 8 < ncols_a);
             lanes_b[j] = HASB ? __builtin_amdgcn_ballot_w64(is_b && cc * 8 < ncols_b) : 0;
             off[j] = (uint32_t)r * (uint32_t)((is_b ? ldb : lda) * 2) + cc * 16;

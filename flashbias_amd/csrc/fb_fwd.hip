@@ -30,10 +30,13 @@ namespace fb {
 
 // VEC: every streamed tensor is 16-byte aligned (base and strides) and d, r are multiples of 8.
 // QB2_: allow two query blocks per wave (the launcher turns it off for small grids).
-template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, bool QB2_ = true>
+// FOLD_: the scores are scale * (q k^T + (q_b / scale) k_b^T), one MFMA chain and no FMA per
+// score for the scale (see the launcher for when that is exact).
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, bool QB2_ = true, bool FOLD_ = false>
 struct FwdCfg {
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
-    static constexpr bool VEC = VEC_, MASK = MASK_;
+    static constexpr bool VEC = VEC_, MASK = MASK_, FOLD = FOLD_;
+    static_assert(!FOLD_ || !MASK_, "the additive mask is not divided by the scale");
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     // query blocks (of 32) per wave: two where the registers allow, so that every key / value
     // fragment read from LDS feeds two blocks and two waves per SIMD carry four softmax streams
@@ -117,6 +120,13 @@ struct FwdLoader {
     uint32_t kdst[C::K_PT], kbdst[C::KB_PT > 0 ? C::KB_PT : 1], vdst[C::V_PT];
     bool kok[C::K_PT], kbok[C::KB_PT > 0 ? C::KB_PT : 1], vok[C::V_PT];
 
+    // Folded scale with r <= 8: columns 8..15 of the bias step hold a second copy of k_b, the
+    // partner of the low parts of q_b / scale in the query operand.
+    static __device__ __forceinline__ bool low_parts(const FwdArgs &a) { return C::FOLD && C::NKR == 1 && a.r <= 8; }
+    static __device__ __forceinline__ int bias_src_chunk(const FwdArgs &a, int ch) {
+        return (low_parts(a) && ch == 1) ? 0 : ch;
+    }
+
     __device__ __forceinline__ void init(const FwdArgs &a, int tid) {
 #pragma unroll
         for (int i = 0; i < C::K_PT; ++i) {
@@ -130,8 +140,9 @@ struct FwdLoader {
         for (int i = 0; i < C::KB_PT; ++i) {
             const int task = tid + i * C::NTHREADS;
             const int row = task % C::BN, ch = task / C::BN;
-            kbok[i] = task < C::KB_TASKS && ch * 8 < a.r;
-            kboff[i] = kbok[i] ? (uint32_t)(row * a.kb.ss + ch * 8) : 0u;
+            const int src = bias_src_chunk(a, ch);
+            kbok[i] = task < C::KB_TASKS && src * 8 < a.r;
+            kboff[i] = kbok[i] ? (uint32_t)(row * a.kb.ss + src * 8) : 0u;
             kbdst[i] = row * C::DKP + 16 * C::NKD + ch * 8;
         }
 #pragma unroll
@@ -172,7 +183,8 @@ struct FwdLoader {
 #pragma unroll
             for (int i = 0; i < C::KB_PT; ++i) {
                 const int task = tid + i * C::NTHREADS;
-                st.kb[i] = load_chunk<C::VEC>(kbbase, a.kb.ss, n0 + task % C::BN, a.Lk, (task / C::BN) * 8, a.r);
+                st.kb[i] = load_chunk<C::VEC>(kbbase, a.kb.ss, n0 + task % C::BN, a.Lk,
+                                              bias_src_chunk(a, task / C::BN) * 8, a.r);
             }
         }
 #pragma unroll
@@ -260,8 +272,11 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
             qr[qb][t] = load_chunk<C::VEC>(qbase, a.q.ss, query, a.Lq, 16 * t + 8 * g, a.d);
         if constexpr (C::NKR > 0) {
 #pragma unroll
-            for (int t = 0; t < C::NKR; ++t)
-                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, 16 * t + 8 * g, a.r);
+            for (int t = 0; t < C::NKR; ++t) {
+                const bool low = FwdLoader<C>::low_parts(a) && g == 1;
+                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, low ? 0 : 16 * t + 8 * g, a.r);
+                if constexpr (C::FOLD) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, FwdLoader<C>::low_parts(a), low);
+            }
         }
 #pragma unroll
         for (int n = 0; n < C::NDV; ++n)
@@ -271,7 +286,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
         m2[qb] = 0.f;
         l_run[qb] = 0.f;
     }
-    constexpr float kLagNat = 8.0f * kLn2; // let the row max run ahead of m_ref by up to 2^8
+    // m_ref and the scores are in natural units, or in units of 1 / scale when the scale is folded
+    const float to_log2 = C::FOLD ? a.scale * kLog2e : kLog2e;
+    const float lag = 8.0f / to_log2; // let the row max run ahead of m_ref by up to 2^8
 
     // causal: tiles past the last query of this workgroup are never visible (:202)
     int k_end = a.Lk;
@@ -403,12 +420,16 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
                                                              sK + (sub * C::BSUB + kb * 32 + c) * C::DKP + 16 * t + 8 * g);
                         if (t < C::NKD)
                             acc = T::mfma(kf, qr[qb][t], acc);
+                        else if (C::FOLD)
+                            acc = T::mfma(kf, qbr[qb][t - C::NKD], acc);
                         else
                             accb = T::mfma(kf, qbr[qb][t - C::NKD], accb);
                     }
+                    if constexpr (!C::FOLD) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        acc[v] = (C::NKR > 0 || C::MASK) ? __builtin_fmaf(acc[v], a.scale, accb[v]) : acc[v] * a.scale;
+                        for (int v = 0; v < 16; ++v)
+                            acc[v] = (C::NKR > 0 || C::MASK) ? __builtin_fmaf(acc[v], a.scale, accb[v]) : acc[v] * a.scale;
+                    }
                     s[kb] = acc;
                 }
                 // ---- -inf for keys past the end and causal-hidden pairs
@@ -430,17 +451,17 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
 #pragma unroll
                     for (int v = (kb == 0 ? 1 : 0); v < 16; ++v) mx = fmaxf(mx, s[kb][v]);
                 mx = half_wave_max(mx);
-                const bool grow = mx > m_ref[qb] + kLagNat; // also true for the first finite score of a row
+                const bool grow = mx > m_ref[qb] + lag; // also true for the first finite score of a row
                 if (__any(grow)) {
                     const float m_new = grow ? mx : m_ref[qb];
-                    const float alpha = grow ? fast_exp2((m_ref[qb] - m_new) * kLog2e) : 1.f; // exp2(-inf) = 0
+                    const float alpha = grow ? fast_exp2((m_ref[qb] - m_new) * to_log2) : 1.f; // exp2(-inf) = 0
                     l_run[qb] *= alpha;
 #pragma unroll
                     for (int n = 0; n < C::NDV; ++n)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) acc_o[qb][n][v] *= alpha;
                     m_ref[qb] = m_new;
-                    m2[qb] = (m_new == -INFINITY) ? 0.f : m_new * kLog2e;
+                    m2[qb] = (m_new == -INFINITY) ? 0.f : m_new * to_log2;
                 }
                 // ---- P^T = exp(S^T - m_ref), row sums (of the fp32 values, :271), O^T += V^T P^T
 #pragma unroll
@@ -450,8 +471,8 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
                         u32x4_t pb;
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
-                            const float p0 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e], kLog2e, -m2[qb]));
-                            const float p1 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e + 1], kLog2e, -m2[qb]));
+                            const float p0 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e], to_log2, -m2[qb]));
+                            const float p1 = fast_exp2(__builtin_fmaf(s[kb][8 * t + 2 * e + 1], to_log2, -m2[qb]));
                             pb[e] = T::pack2(p0, p1);
                             l_run[qb] += p0 + p1;
                         }
@@ -481,7 +502,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
         const float l = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
         const float inv = 1.f / l;
         if (query < a.Lq) {
-            if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref[qb] + __builtin_amdgcn_logf(l) * kLn2;
+            if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref[qb] * (C::FOLD ? a.scale : 1.f) + __builtin_amdgcn_logf(l) * kLn2;
             uint16_t *orow = obase + (int64_t)query * a.o.ss;
 #pragma unroll
             for (int n = 0; n < C::NDV; ++n)
@@ -503,9 +524,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
     }
 }
 
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool QB2>
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool QB2, bool FOLD>
 static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
-    typedef FwdCfg<T, NKD, NKR, NDV, VEC, MASK, QB2> C;
+    typedef FwdCfg<T, NKD, NKR, NDV, VEC, MASK, QB2, FOLD> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_kernel<T, C>;
@@ -523,14 +544,14 @@ static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
 // workgroups (three under a causal mask, whose tiles differ in length); below that, 128-query
 // workgroups at three waves per SIMD fill the chip better (measured: 35 % faster at a quarter
 // of that grid, 10 % slower at twice it).
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK>
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_fwd_vec(const FwdArgs &a, hipStream_t stream) {
     if constexpr (FwdCfg<T, NKD, NKR, NDV, VEC, MASK, true>::QB == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
         if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus())
-            return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, false>(a, stream);
+            return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, false, FOLD>(a, stream);
     }
-    return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, true>(a, stream);
+    return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, true, FOLD>(a, stream);
 }
 
 template <class T, int NKD, int NKR, int NDV>
@@ -543,6 +564,9 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
     if (a.mask.type)
         return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    if constexpr (NKR <= 2) {
+        if (vec && fold_scale_ok<T>(a.scale, a.r)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
+    }
     return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, false>(a, stream)
                : launch_fwd_vec<T, NKD, NKR, NDV, false, false>(a, stream);
 }

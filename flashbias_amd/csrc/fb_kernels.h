@@ -1,5 +1,6 @@
 // Host-visible kernel argument blocks and launchers (implemented in fb_fwd.hip / fb_bwd.hip).
 #pragma once
+#include <cmath>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -56,5 +57,20 @@ inline int num_cus() {
 inline int steps_pow2(int n16) { return n16 <= 1 ? 1 : n16 <= 2 ? 2 : n16 <= 4 ? 4 : 8; }
 inline int nkd_of(int d) { return steps_pow2((d + 15) / 16); }
 inline int nkr_of(int r) { return r == 0 ? 0 : steps_pow2((r + 15) / 16); }
+
+// Whether a kernel may compute scale * (q k^T + (q_b / scale) k_b^T) in one MFMA chain instead of
+// scale * q k^T + q_b k_b^T (one FMA per score less) and still match the fp32 scaling of the
+// reference: always without factors; with factors only for an element type with the exponent
+// range of fp32 (the division cannot overflow) and either a power-of-two scale (the division is
+// exact) or r <= 8 (the low-order half of q_b / scale travels in the unused half of the 16-wide
+// MFMA step, which leaves a relative error of 2^-17 in the bias product).
+template <class T>
+inline bool fold_scale_ok(float scale, int r) {
+    if (!(scale > 1e-30f && scale < 1e30f)) return false;
+    if (r == 0) return true;
+    if (!T::kWideRange) return false;
+    int e;
+    return r <= 8 || std::frexp(scale, &e) == 0.5f;
+}
 
 } // namespace fb

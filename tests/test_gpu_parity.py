@@ -79,6 +79,47 @@ def test_large_head_dim_and_rank_together(gpu_device, d, r, causal):
     _case(gpu_device, 2, 333, 401, 2, d, r, torch.bfloat16, causal, seed=17)
 
 
+@pytest.mark.parametrize("d,r,scale", [(32, 8, None), (32, 8, 0.25), (32, 8, 0.29), (32, 8, 3.0), (64, 16, None),
+                                       (64, 32, 0.5), (64, 24, 0.3), (128, 8, None), (32, 0, None), (32, 0, 0.7),
+                                       (32, 8, -0.2), (64, 0, -0.125)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_scale_folded_into_the_contraction(gpu_device, d, r, scale, dtype):
+    """Where it is exact (no factors; bf16 factors with a power-of-two scale or r <= 8) the kernels
+    compute scale * (q k^T + (q_b / scale) k_b^T) in one MFMA chain; elsewhere (fp16 factors, other
+    scales at larger ranks, scales <= 0) they scale the fp32 q k^T product.  Both against the
+    oracle, with factors large enough (bias entries ~ N(0, 10^2)) that the bias dominates."""
+    B, Lq, Lk, H = 2, 300, 330, 2
+    q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, dtype, seed=23)
+    if r:
+        qb = (qb.float() * 10.0 * math.sqrt(r)).to(dtype)  # entries of q_b k_b^T: std 1 / sqrt(r) before
+    for causal in (False, True):
+        ref = oracle(q, k, v, qb, kb, None, causal, scale, do)
+        got = run_gpu(flash_bias_func, q, k, v, qb, kb, None, causal, scale, do, gpu_device)
+        _gate(got, ref, dtype)
+
+
+@pytest.mark.parametrize("scale", [None, 0.25, 0.29, 0.3])
+def test_infinite_factor_column(gpu_device, scale):
+    """A key-padding column in the factors themselves (q_b column of ones against a k_b column of
+    0 / -inf): with the scale folded into q_b or k_b as high and low parts, both parts must give
+    the same infinity (scales whose reciprocal rounds up, rounds down, and is exact in bf16)."""
+    B, Lq, Lk, H, d, r = 2, 200, 264, 2, 32, 8
+    q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, torch.bfloat16, seed=29)
+    qb[..., r - 1] = 1.0
+    kb[..., r - 1] = 0.0
+    kb[:, Lk - 70:, :, r - 1] = float("-inf")
+    kb[0, 3, :, r - 1] = float("-inf")
+    ref = oracle(q, k, v, qb, kb, None, False, scale, do)
+    got = run_gpu(flash_bias_func, q, k, v, qb, kb, None, False, scale, do, gpu_device)
+    # the gradient of that q_b column is a sum with 0 * inf terms in any arithmetic: compare the rest
+    for name, g, w in zip(NAMES, got, [ref[0]] + list(ref[2:])):
+        if name == "dq_bias":
+            g, w = g[..., :r - 1], w[..., :r - 1]
+        assert torch.isfinite(g).all(), name
+        err, rel = errors(g, w)
+        assert (err <= O_TOL[torch.bfloat16]) if name == "o" else (rel <= GRAD_TOL), (name, err, rel)
+
+
 @pytest.mark.parametrize("Lq,Lk", [(1, 1), (1, 257), (75, 117), (117, 75), (129, 64), (64, 129), (255, 255)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_ragged_lengths(gpu_device, Lq, Lk, causal):
