@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
 # HBM bytes of one dk/dv launch at the headline shape: rocprofv3 FETCH_SIZE (x2.0, calibrated on a copy of
 # known size) + WRITE_SIZE, see profiles/headline_fwd_bwd_kernels.md; a counter figure, not measured live
-DKV_HBM_BYTES = 1.77e8
+DKV_HBM_BYTES = 1.73e8
 PEAK_HBM_GBS = 8000.0
 
 

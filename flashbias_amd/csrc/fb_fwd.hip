@@ -16,12 +16,15 @@
 // zero-padded to 16-wide MFMA steps.
 //
 // Softmax scale: the reference multiplies the fp32 q k^T accumulator by the scale and never
-// scales the bias product (flash_bias_triton.py:246-256).  Same here: q k^T and q_b k_b^T are two
-// separate (and therefore independent, shorter) MFMA chains, joined by one fp32 FMA per score.
-// Measured on MI355X this beats folding the scale into the query operand (which needs a second,
-// low-order MFMA per step): the matrix pipe is the scarcer resource when two waves share a SIMD.
+// scales the bias product (flash_bias_triton.py:246-256).  General case here: q k^T and q_b k_b^T
+// are two separate (and therefore independent, shorter) MFMA chains, joined by one fp32 FMA per
+// score.  (Folding the scale into the query operand needs a second, low-order MFMA per step and
+// measured slower: the matrix pipe is the scarcer resource when two waves share a SIMD.)
+// FOLD instantiations (no mask; no factors, or bf16 factors with a power-of-two scale or r <= 8,
+// see fold_scale_ok) instead divide q_b by the scale once, keep the scores in units of 1 / scale
+// in one MFMA chain, and apply the scale inside the FMA that feeds exp2: one FMA per score less.
 //
-// Per score the VALU does: fma (scale), max3, fma + exp2, convert, add (row sum); the running
+// Per score the VALU does: [fma (scale),] max3, fma + exp2, convert, add (row sum); the running
 // reference of the softmax only moves when a row maximum grows by more than 2^8 (then
 // p <= 256, exact enough in fp32 / 16-bit), so the accumulator rescale is rare.
 #include "fb_kernels.h"
