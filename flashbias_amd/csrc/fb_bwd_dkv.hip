@@ -602,7 +602,7 @@ static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
         return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_dkv_vec<T, NKD, NKR, NDV, false, true>(a, stream);
     if constexpr (NKR <= 2) {
-        if (vec && fold_scale_ok<T>(a.scale, a.r)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
+        if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lq)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
     }
     return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, false>(a, stream)
                : launch_dkv_vec<T, NKD, NKR, NDV, false, false>(a, stream);

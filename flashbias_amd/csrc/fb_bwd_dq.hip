@@ -473,7 +473,7 @@ static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
     if (a.mask.type)
         return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
     if constexpr (NKR <= 2) {
-        if (vec && fold_scale_ok<T>(a.scale, a.r)) return launch_dq_vec<T, NKD, NKR, true, false, true>(a, stream);
+        if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_dq_vec<T, NKD, NKR, true, false, true>(a, stream);
     }
     return vec ? launch_dq_vec<T, NKD, NKR, true, false>(a, stream) : launch_dq_vec<T, NKD, NKR, false, false>(a, stream);
 }

@@ -568,7 +568,7 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
         return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
     if constexpr (NKR <= 2) {
-        if (vec && fold_scale_ok<T>(a.scale, a.r)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
+        if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
     }
     return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, false>(a, stream)
                : launch_fwd_vec<T, NKD, NKR, NDV, false, false>(a, stream);

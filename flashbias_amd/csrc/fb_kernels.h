@@ -63,12 +63,15 @@ inline int nkr_of(int r) { return r == 0 ? 0 : steps_pow2((r + 15) / 16); }
 // reference: always without factors; with factors only for an element type with the exponent
 // range of fp32 (the division cannot overflow) and either a power-of-two scale (the division is
 // exact) or r <= 8 (the low-order half of q_b / scale travels in the unused half of the 16-wide
-// MFMA step, which leaves a relative error of 2^-16 in the bias product).
+// MFMA step, which leaves a relative error of 2^-16 in the bias product).  `len` is the length
+// of the loop a workgroup runs (keys in the forward and dq kernels, queries in dk/dv): dividing
+// the resident factor costs about as much as the FMAs of 256 loop positions, so short loops keep
+// the FMA.
 template <class T>
-inline bool fold_scale_ok(float scale, int r) {
+inline bool fold_scale_ok(float scale, int r, int len) {
     if (!(scale > 1e-6f && scale < 1e6f)) return false; // (also false for NaN; keeps 1 / scale and scale * score well inside fp32)
     if (r == 0) return true;
-    if (!T::kWideRange) return false;
+    if (!T::kWideRange || len < 512) return false;
     int e;
     return r <= 8 || std::frexp(scale, &e) == 0.5f;
 }

@@ -86,9 +86,10 @@ def test_large_head_dim_and_rank_together(gpu_device, d, r, causal):
 def test_scale_folded_into_the_contraction(gpu_device, d, r, scale, dtype):
     """Where it is exact (no factors; bf16 factors with a power-of-two scale or r <= 8) the kernels
     compute scale * (q k^T + (q_b / scale) k_b^T) in one MFMA chain; elsewhere (fp16 factors, other
-    scales at larger ranks, scales <= 0) they scale the fp32 q k^T product.  Both against the
-    oracle, with factors large enough (bias entries ~ N(0, 10^2)) that the bias dominates."""
-    B, Lq, Lk, H = 2, 300, 330, 2
+    scales at larger ranks, scales <= 0, and loops shorter than 512 with factors) they scale the
+    fp32 q k^T product.  Both against the oracle, with factors large enough (bias entries
+    ~ N(0, 10^2)) that the bias dominates."""
+    B, Lq, Lk, H = 2, 530, 600, 2
     q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, dtype, seed=23)
     if r:
         qb = (qb.float() * 10.0 * math.sqrt(r)).to(dtype)  # entries of q_b k_b^T: std 1 / sqrt(r) before
@@ -103,7 +104,7 @@ def test_infinite_factor_column(gpu_device, scale):
     """A key-padding column in the factors themselves (q_b column of ones against a k_b column of
     0 / -inf): with the scale folded into q_b or k_b as high and low parts, both parts must give
     the same infinity (scales whose reciprocal rounds up, rounds down, and is exact in bf16)."""
-    B, Lq, Lk, H, d, r = 2, 200, 264, 2, 32, 8
+    B, Lq, Lk, H, d, r = 2, 520, 584, 2, 32, 8
     q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, torch.bfloat16, seed=29)
     qb[..., r - 1] = 1.0
     kb[..., r - 1] = 0.0
