@@ -71,11 +71,13 @@ def test_ranks(gpu_device, r):
     _case(gpu_device, 1, 160, 224, 2, 32, r, torch.bfloat16, False)
 
 
-@pytest.mark.parametrize("d,r", [(64, 64), (128, 64), (64, 128), (16, 128), (128, 128), (72, 24)])
+@pytest.mark.parametrize("d,r", [(64, 64), (128, 64), (64, 128), (16, 128), (128, 128), (72, 24), (128, 8), (96, 32),
+                                 (128, 0)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_large_head_dim_and_rank_together(gpu_device, d, r, causal):
-    """Instantiations with many contraction steps: their register budget, LDS footprint and (head
-    dim 128) three-pass dk/dv differ from the small configurations."""
+    """Instantiations with many contraction steps: their register budget, LDS footprint, (head dim
+    128) multi-pass dk/dv and (head dims above 64, rank <= 32) 32-key tiles in the dq kernel differ
+    from the small configurations."""
     _case(gpu_device, 2, 333, 401, 2, d, r, torch.bfloat16, causal, seed=17)
 
 
