@@ -25,11 +25,11 @@
 
 namespace fb {
 
-// PART: 0 = dv, dk and dk_bias in one pass; 1 = dv only; 3 / 4 = the lower / upper half of the
-// 32-row blocks of [dk | dk_bias] only; 6 = dv and the lower half.  Head dims above 64 run as two
-// launches (6, 4) while the accumulators of pass 6 fit 256 registers (ranks up to 32), else as
-// three (1, 3, 4), with 32-query steps: each pass keeps its accumulators in registers and its LDS
-// stages small enough for two waves per SIMD, which is worth recomputing S.
+// PART: 0 = dv, dk and dk_bias in one pass; 1 = dv only; 2 = [dk | dk_bias] only; 3 / 4 = the
+// lower / upper half of the 32-row blocks of [dk | dk_bias] only.  Head dims above 64 run as two
+// launches (1, 2) while the accumulators of pass 2 fit 256 registers (ranks up to 32, no mask),
+// else as three (1, 3, 4), with 32-query steps: each pass keeps its accumulators in registers and
+// its LDS stages small enough for two waves per SIMD, which is worth recomputing S.
 // FOLD_: the scores are scale * (q k^T + q_b (k_b / scale)^T), no multiply per score for the scale
 // (the launcher says when that is exact).
 template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, int PART_ = 0, bool FOLD_ = false>
@@ -41,12 +41,12 @@ struct DkvCfg {
     static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8; }
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
-    static constexpr bool DO_DV = PART_ <= 1 || PART_ == 6, DO_DK = PART_ != 1;
+    static constexpr bool DO_DV = PART_ <= 1, DO_DK = PART_ != 1;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dK | dK_b]^T
     // ... of which this instantiation accumulates [MB0, MB1)
-    static constexpr int MB0 = PART_ == 4 ? MB / 2 : 0, MB1 = PART_ == 1 ? 0 : (PART_ == 3 || PART_ == 6) ? MB / 2 : MB;
+    static constexpr int MB0 = PART_ == 4 ? MB / 2 : 0, MB1 = PART_ == 1 ? 0 : PART_ == 3 ? MB / 2 : MB;
     static constexpr int KBW = 1; // key blocks per wave
     static constexpr int BN = 32 * KBW * NWAVES;              // keys per workgroup
     static constexpr int QBLK = PART_ == 0 ? 2 : 1, BMQ = 32 * QBLK; // queries per step
@@ -576,10 +576,13 @@ static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_dkv_vec(const BwdArgs &a, hipStream_t stream) {
     if constexpr (NKD > 4 && VEC) {
-        if constexpr (NKR <= 2 && !MASK) { // two passes: measured 10-18 % faster than three
-            const hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 6, FOLD>(a, stream);
+        if constexpr (NKR <= 2 && !MASK) {
+            // two passes, dv and then all of [dk | dk_bias]: 44 MFMAs per 32 x 32 block (three passes: 61;
+            // dv with the lower half of dk, then the upper half: 52, measured 15-24 % slower than this)
+            const hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 1, FOLD>(a, stream);
             if (e != hipSuccess) return e;
-        } else {
+            return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 2, FOLD>(a, stream);
+        } else { // larger ranks and masked calls: all of dk would spill at 256 registers
             hipError_t e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 1, FOLD>(a, stream);
             if (e != hipSuccess) return e;
             e = launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 3, FOLD>(a, stream);
