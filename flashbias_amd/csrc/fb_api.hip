@@ -233,10 +233,17 @@ int fb_bwd_dq(const fb_params *p, void *stream) {
 }
 
 int fb_bwd(const fb_params *p, void *stream) {
-    int rc = fb_bwd_preprocess(p, stream);
+    // Two launches: the dq kernel computes delta for its own queries on the way (each query belongs
+    // to exactly one of its workgroups) and leaves the statistics in the scratch buffer for the
+    // dk/dv kernel.  The three phases above stay callable one by one.
+    const int rc = fb_check(p, 1);
     if (rc) return rc;
-    if ((rc = fb_bwd_dkv(p, stream))) return rc;
-    return fb_bwd_dq(p, stream);
+    fb::BwdArgs a = bwd_args(p);
+    a.stats_here = 1;
+    const int rc2 = launched(fb::launch_bwd_dq(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd_dq");
+    if (rc2) return rc2;
+    a.stats_here = 0;
+    return launched(fb::launch_bwd_dkv(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd_dkv");
 }
 
 } // extern "C"

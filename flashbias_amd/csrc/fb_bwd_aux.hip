@@ -30,8 +30,8 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a) {
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                acc += T::to_float((uint16_t)(x[e] & 0xffffu)) * T::to_float((uint16_t)(y[e] & 0xffffu));
-                acc += T::to_float((uint16_t)(x[e] >> 16)) * T::to_float((uint16_t)(y[e] >> 16));
+                acc = __builtin_fmaf(T::to_float((uint16_t)(x[e] & 0xffffu)), T::to_float((uint16_t)(y[e] & 0xffffu)), acc);
+                acc = __builtin_fmaf(T::to_float((uint16_t)(x[e] >> 16)), T::to_float((uint16_t)(y[e] >> 16)), acc);
             }
         }
         a.delta[rix] = -acc;
@@ -65,8 +65,8 @@ __global__ __launch_bounds__(256) void bwd_preprocess_chunks_kernel(const BwdArg
             const u32x4_t y = *reinterpret_cast<const u32x4_t *>(drow + c * 8);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                acc += T::to_float((uint16_t)(x[e] & 0xffffu)) * T::to_float((uint16_t)(y[e] & 0xffffu));
-                acc += T::to_float((uint16_t)(x[e] >> 16)) * T::to_float((uint16_t)(y[e] >> 16));
+                acc = __builtin_fmaf(T::to_float((uint16_t)(x[e] & 0xffffu)), T::to_float((uint16_t)(y[e] & 0xffffu)), acc);
+                acc = __builtin_fmaf(T::to_float((uint16_t)(x[e] >> 16)), T::to_float((uint16_t)(y[e] >> 16)), acc);
             }
         }
 #pragma unroll

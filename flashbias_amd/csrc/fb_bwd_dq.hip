@@ -223,9 +223,45 @@ bwd_dq_kernel(const BwdArgs a) {
         }
         const bool ok = query < a.Lq;
         const int64_t sidx = (int64_t)bh * a.Lq + (ok ? query : a.Lq - 1);
-        // the preprocess step left -delta and lse * log2(e) in the scratch buffer
-        lse2[qb] = ok ? a.delta[(int64_t)a.B * a.H * a.Lq + sidx] : INFINITY; // rows past the end: P = exp2(-inf) = 0
-        const float nd = ok ? a.delta[sidx] : 0.f;
+        float nd, l2;
+        if (a.stats_here) {
+            // delta = rowsum(o * dO) of this lane's query (flash_bias_triton.py:358-400) from the dO
+            // chunks it holds and the same chunks of o; the other half of the channels is with lane ^ 32.
+            // -delta and lse * log2(e) also go to the scratch buffer, for the dk/dv kernel that follows.
+            const uint16_t *obase = a.o.ptr + b * a.o.sb + h * a.o.sh;
+            // (summed in the order of the preprocess kernel: per 8-channel chunk, then a pairwise tree
+            // over the chunks, so that both ways of running the backward give the same bits)
+            float cs[C::NKD];
+#pragma unroll
+            for (int t = 0; t < C::NKD; ++t) {
+                const u32x4_t oc = load_chunk<C::VEC>(obase, a.o.ss, query, a.Lq, 16 * t + 8 * g, a.d);
+                float acc1 = 0.f;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    acc1 = __builtin_fmaf(T::to_float((uint16_t)(oc[e] & 0xffffu)),
+                                          T::to_float((uint16_t)(dor[qb][t][e] & 0xffffu)), acc1);
+                    acc1 = __builtin_fmaf(T::to_float((uint16_t)(oc[e] >> 16)), T::to_float((uint16_t)(dor[qb][t][e] >> 16)),
+                                          acc1);
+                }
+                cs[t] = acc1 + __shfl_xor(acc1, 32, 64); // chunks 2t and 2t + 1
+            }
+#pragma unroll
+            for (int m = 1; m < C::NKD; m <<= 1)
+#pragma unroll
+                for (int t = 0; t + m < C::NKD; t += 2 * m) cs[t] += cs[t + m];
+            const float part = cs[0];
+            nd = ok ? -part : 0.f;
+            l2 = ok ? a.lse[sidx] * kLog2e : INFINITY;
+            if (ok && g == 0) {
+                a.delta[sidx] = nd;
+                a.delta[(int64_t)a.B * a.H * a.Lq + sidx] = l2;
+            }
+        } else {
+            // the preprocess step left -delta and lse * log2(e) in the scratch buffer
+            l2 = ok ? a.delta[(int64_t)a.B * a.H * a.Lq + sidx] : INFINITY;
+            nd = ok ? a.delta[sidx] : 0.f;
+        }
+        lse2[qb] = l2; // rows past the end: P = exp2(-inf) = 0
 #pragma unroll
         for (int v = 0; v < 16; ++v) negd[qb][v] = nd;
 #pragma unroll
@@ -480,7 +516,7 @@ static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
     const int64_t lim = (int64_t)1 << 24;
     const bool vec = a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.d % 8 == 0 &&
                      (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.r % 8 == 0)) && a.k.ss < lim && a.v.ss < lim &&
-                     (a.r == 0 || a.kb.ss < lim);
+                     (a.r == 0 || a.kb.ss < lim) && (!a.stats_here || a.o.vec_ok);
     if (a.mask.type)
         return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
     if constexpr (NKR <= 2) {

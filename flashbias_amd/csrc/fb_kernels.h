@@ -29,6 +29,7 @@ struct BwdArgs {
     float scale;
     int ntiles_n; // key tiles per (batch, head), dk/dv kernel
     int ntiles_m; // query tiles per (batch, head), dq kernel
+    int stats_here; // dq kernel: compute -delta and lse * log2(e) itself (and store them) instead of reading them
 };
 
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.
