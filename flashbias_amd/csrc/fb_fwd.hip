@@ -544,14 +544,16 @@ static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
 }
 
 // Two query blocks per wave (256 queries per workgroup) pay once every compute unit has two such
-// workgroups (three under a causal mask, whose tiles differ in length); below that, 128-query
-// workgroups at three waves per SIMD fill the chip better (measured: 35 % faster at a quarter
-// of that grid, 10 % slower at twice it).
+// workgroups; below that, 128-query workgroups at three waves per SIMD fill the chip better
+// (measured: 35 % faster at a quarter of that grid, 10 % slower at twice it).  Under a causal mask
+// the workgroups differ in length and the short ones leave the chip part empty towards the end:
+// the small workgroups stay ahead up to seven per compute unit (B1 H50 d32: 13 % faster at
+// L=4096, 5 % at L=8192, equal at L=16384).
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_fwd_vec(const FwdArgs &a, hipStream_t stream) {
     if constexpr (FwdCfg<T, NKD, NKR, NDV, VEC, MASK, true>::QB == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus())
+        if (wgs < (int64_t)(a.causal ? 7 : 2) * num_cus())
             return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, false, FOLD>(a, stream);
     }
     return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, true, FOLD>(a, stream);
