@@ -101,14 +101,18 @@ size_t fb_bwd_workspace_bytes(const fb_params *p);
  * o = softmax(scale q k^T + q_bias k_bias^T + mask) v and lse. */
 int fb_fwd(const fb_params *p, void *stream);
 
-/* Replaces _flash_attn_backward (flash_bias_triton.py:1197-1342): runs the three phases
- * below in order on the stream.  Unlike the reference there is no fp32 dq_accum buffer, no
+/* Replaces _flash_attn_backward (flash_bias_triton.py:1197-1342).  Two launches on the stream: the
+ * query-stationary kernel (dq, dq_bias), which also forms delta = rowsum(o * dout) for its own
+ * queries and leaves -delta and lse * log2(e) in the scratch buffer, then the key-stationary kernel
+ * (dk, dv, dk_bias) that reads them.  The results are bit-identical to the three phases below
+ * called one by one.  Unlike the reference there is no fp32 dq_accum buffer, no
  * atomics and no final cast (:1212-1219, :1340-1342): dq and dq_bias are accumulated in
  * registers by a query-stationary kernel and written once, so every gradient is
  * bit-reproducible. */
 int fb_bwd(const fb_params *p, void *stream);
 
-/* The phases of fb_bwd, exported so that a harness can time them separately.
+/* The backward in three phases, exported so that a harness can time them separately (call them in
+ * this order: the two main kernels read what the preprocess wrote).
  *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400); fills the
  *                      scratch with -delta (first B*H*Lq floats) and lse * log2(e) (next B*H*Lq)
  *   fb_bwd_dkv:        recompute P from lse; dk, dv, dk_bias, one workgroup per key tile
