@@ -226,6 +226,7 @@ def report(args):
     cases += [(f"alibi causal L={L}", lambda L=L: workloads.alibi(L), False) for L in (2048, 4096, 8192)]
     cases += [("swin 4096x256 r16", lambda: workloads.swin(), False), ("pde N=32768 r5", lambda: workloads.pde(), False),
               ("pairformer 768 r32", lambda: workloads.pairformer(), False),
+              ("swin 4096x256 r16 + shifted-window mask", lambda: workloads.swin(shifted_types=64), None),
               ("sweep L=4096 + vector mask", lambda: workloads.masked(4096, "vector"), None),
               ("sweep L=4096 + matrix mask", lambda: workloads.masked(4096, "matrix"), None)]
     # other head dims and ranks at L=8192, and a causal language-model-like shape

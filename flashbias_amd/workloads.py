@@ -60,15 +60,26 @@ def alibi(L, H=50, d=32, dtype=torch.bfloat16, seed=0):
     return _pack(q, k, v, do, qb, kb, True, 1.0 / math.sqrt(d))
 
 
-def swin(windows=4096, window=16, H=16, d=32, r=16, dtype=torch.bfloat16, seed=0):
+def swin(windows=4096, window=16, H=16, d=32, r=16, dtype=torch.bfloat16, seed=0, shifted_types=0):
     """Swin-V2 style windowed attention: `windows` windows of window^2 tokens, per-head bias
-    table factored by truncated SVD and shared by all windows (broadcast over batch)."""
+    table factored by truncated SVD and shared by all windows (broadcast over batch).
+    shifted_types > 0 adds the additive mask of a shifted-window block the way the reference
+    hands it to the operator (2_Vision_Transformer/swin_transformer_v2.py:171-173, :190-203):
+    one 0 / -100 matrix per window type, repeated over the images into (windows, 1, n, n)."""
     g = torch.Generator().manual_seed(seed)
     n = window * window
     q, k, v, do = _qkv(windows, n, n, H, d, g, dtype)
     table = factors.swin_v2_bias_table(window, H, seed)
     qb, kb, rel = factors.svd_factors(table, r, dtype)
-    return _pack(q, k, v, do, qb, kb, False, 1.0 / math.sqrt(d), bias_table=table, bias_rel_error=rel)
+    w = _pack(q, k, v, do, qb, kb, False, 1.0 / math.sqrt(d), bias_table=table, bias_rel_error=rel)
+    if shifted_types:
+        assert windows % shifted_types == 0
+        # tokens of a shifted window fall into up to four regions; pairs from different regions get -100
+        region = torch.randint(0, 4, (shifted_types, n), generator=g)
+        region[0] = 0  # (the unshifted interior windows see everything)
+        m = (region[:, :, None] != region[:, None, :]).to(dtype) * -100.0
+        w["mask"] = m.unsqueeze(1).unsqueeze(0).repeat(windows // shifted_types, 1, 1, 1, 1).reshape(windows, 1, n, n)
+    return w
 
 
 def pde(N=32768, H=8, d=32, alpha=10.0, dtype=torch.bfloat16, seed=0):

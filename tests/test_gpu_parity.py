@@ -406,8 +406,9 @@ def test_random_shapes(gpu_device, idx):
 
 # ------------------------------------------------------------------ named workloads (reduced)
 def _run_workload(gpu_device, w, dtype, skip=()):
-    ref = oracle(w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], None, w["causal"], w["softmax_scale"], w["do"])
-    got = run_gpu(flash_bias_func, w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], None, w["causal"],
+    mask = w.get("mask")
+    ref = oracle(w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], mask, w["causal"], w["softmax_scale"], w["do"])
+    got = run_gpu(flash_bias_func, w["q"], w["k"], w["v"], w["q_bias"], w["k_bias"], mask, w["causal"],
                   w["softmax_scale"], w["do"], gpu_device)
     _gate(got, ref, dtype, skip)
     return got, ref
@@ -465,6 +466,14 @@ def test_workload_swin(gpu_device):
     exact = eager.attention_eager(w["q"].float(), w["k"].float(), w["v"].float(), w["softmax_scale"],
                                   w["bias_table"][None].expand(8, -1, -1, -1))
     assert (got[0] - exact).abs().max() < 0.1
+
+
+def test_workload_swin_shifted_windows(gpu_device):
+    """The same windows with the 0 / -100 matrix mask of a shifted-window block, one matrix per
+    window type repeated over the images and broadcast over the heads."""
+    w = workloads.swin(windows=8, shifted_types=4)
+    assert w["mask"].shape == (8, 1, 256, 256)
+    _run_workload(gpu_device, w, torch.bfloat16)
 
 
 def test_workload_pde(gpu_device):
