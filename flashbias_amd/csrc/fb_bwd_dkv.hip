@@ -38,7 +38,7 @@ struct DkvCfg {
     static_assert(!FOLD_ || (VEC_ && !MASK_), "folded scale: direct loader, no additive mask");
     // folded scale with r <= 8: the Q_b columns 8..15 of a step hold a second copy of q_b, the
     // partner of the low parts of k_b / scale in the key operand
-    static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8; }
+    static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8 && a.scale != 1.f; }
     static constexpr int NKD = NKD_, NKR = NKR_, NDV = NDV_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr bool DO_DV = PART_ <= 1, DO_DK = PART_ != 1;
@@ -280,7 +280,7 @@ bwd_dkv_kernel(const BwdArgs a) {
             else if constexpr (C::NKR > 0) {
                 const bool low = C::low_parts(a) && g == 1;
                 kreg[kb][t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, low ? 0 : 16 * (t - C::NKD) + 8 * g, a.r);
-                if constexpr (C::FOLD) kreg[kb][t] = fold_scale_chunk<T>(kreg[kb][t], 1.f / a.scale, C::low_parts(a), low);
+                if (C::FOLD && a.scale != 1.f) kreg[kb][t] = fold_scale_chunk<T>(kreg[kb][t], 1.f / a.scale, C::low_parts(a), low);
             }
         }
         if constexpr (C::DO_DK) {

@@ -31,7 +31,7 @@ struct DqCfg {
     static_assert(!FOLD_ || (VEC_ && !MASK_), "folded scale: direct loader, no additive mask");
     // folded scale with r <= 8: the K_b columns 8..15 of a tile hold a second copy of k_b, the
     // partner of the low parts of q_b / scale in the query operand
-    static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8; }
+    static __device__ __forceinline__ bool low_parts(const BwdArgs &a) { return FOLD_ && NKR_ == 1 && a.r <= 8 && a.scale != 1.f; }
     static constexpr int NKD = NKD_, NKR = NKR_;
     static constexpr bool VEC = VEC_, MASK = MASK_;
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
@@ -218,7 +218,7 @@ bwd_dq_kernel(const BwdArgs a) {
             for (int t = 0; t < C::NKR; ++t) {
                 const bool low = C::low_parts(a) && g == 1;
                 qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, low ? 0 : 16 * t + 8 * g, a.r);
-                if constexpr (C::FOLD) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, C::low_parts(a), low);
+                if (C::FOLD && a.scale != 1.f) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, C::low_parts(a), low);
             }
         }
         const bool ok = query < a.Lq;

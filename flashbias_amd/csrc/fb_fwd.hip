@@ -125,7 +125,7 @@ struct FwdLoader {
 
     // Folded scale with r <= 8: columns 8..15 of the bias step hold a second copy of k_b, the
     // partner of the low parts of q_b / scale in the query operand.
-    static __device__ __forceinline__ bool low_parts(const FwdArgs &a) { return C::FOLD && C::NKR == 1 && a.r <= 8; }
+    static __device__ __forceinline__ bool low_parts(const FwdArgs &a) { return C::FOLD && C::NKR == 1 && a.r <= 8 && a.scale != 1.f; }
     static __device__ __forceinline__ int bias_src_chunk(const FwdArgs &a, int ch) {
         return (low_parts(a) && ch == 1) ? 0 : ch;
     }
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
             for (int t = 0; t < C::NKR; ++t) {
                 const bool low = FwdLoader<C>::low_parts(a) && g == 1;
                 qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, low ? 0 : 16 * t + 8 * g, a.r);
-                if constexpr (C::FOLD) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, FwdLoader<C>::low_parts(a), low);
+                if (C::FOLD && a.scale != 1.f) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, FwdLoader<C>::low_parts(a), low);
             }
         }
 #pragma unroll

@@ -67,11 +67,13 @@ inline int nkr_of(int r) { return r == 0 ? 0 : steps_pow2((r + 15) / 16); }
 // MFMA step, which leaves a relative error of 2^-16 in the bias product).  `len` is the length
 // of the loop a workgroup runs (keys in the forward and dq kernels, queries in dk/dv): dividing
 // the resident factor costs about as much as the FMAs of 256 loop positions, so short loops keep
-// the FMA.
+// the FMA.  A scale of exactly 1 (what the reference's Swin and AlphaFold3 blocks pass, having
+// scaled q themselves: swin_transformer_v2.py:178-203, primitives.py:636-643) needs no division
+// at all: folded for every element type and length, the factors used as they are.
 template <class T>
 inline bool fold_scale_ok(float scale, int r, int len) {
     if (!(scale > 1e-6f && scale < 1e6f)) return false; // (also false for NaN; keeps 1 / scale and scale * score well inside fp32)
-    if (r == 0) return true;
+    if (r == 0 || scale == 1.f) return true;
     if (!T::kWideRange || len < 512) return false;
     int e;
     return r <= 8 || std::frexp(scale, &e) == 0.5f;

@@ -83,10 +83,12 @@ def test_large_head_dim_and_rank_together(gpu_device, d, r, causal):
 
 @pytest.mark.parametrize("d,r,scale", [(32, 8, None), (32, 8, 0.25), (32, 8, 0.29), (32, 8, 3.0), (64, 16, None),
                                        (64, 32, 0.5), (64, 24, 0.3), (128, 8, None), (32, 0, None), (32, 0, 0.7),
-                                       (32, 8, -0.2), (64, 0, -0.125)])
+                                       (32, 8, -0.2), (64, 0, -0.125), (32, 8, 1.0), (32, 16, 1.0), (64, 32, 1.0),
+                                       (128, 8, 1.0)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_scale_folded_into_the_contraction(gpu_device, d, r, scale, dtype):
-    """Where it is exact (no factors; bf16 factors with a power-of-two scale or r <= 8) the kernels
+    """Where it is exact (no factors; a scale of exactly 1, which leaves the factors as they are,
+    for both element types; bf16 factors with a power-of-two scale or r <= 8) the kernels
     compute scale * (q k^T + (q_b / scale) k_b^T) in one MFMA chain; elsewhere (fp16 factors, other
     scales at larger ranks, scales <= 0, and loops shorter than 512 with factors) they scale the
     fp32 q k^T product.  Both against the oracle, with factors large enough (bias entries
@@ -101,7 +103,7 @@ def test_scale_folded_into_the_contraction(gpu_device, d, r, scale, dtype):
         _gate(got, ref, dtype)
 
 
-@pytest.mark.parametrize("scale", [None, 0.25, 0.29, 0.3])
+@pytest.mark.parametrize("scale", [None, 0.25, 0.29, 0.3, 1.0])
 def test_infinite_factor_column(gpu_device, scale):
     """A key-padding column in the factors themselves (q_b column of ones against a k_b column of
     0 / -inf): with the scale folded into q_b or k_b as high and low parts, both parts must give
