@@ -309,6 +309,8 @@ bwd_dq_kernel(const BwdArgs a) {
     __syncthreads();
 
     int cur = 0; // stage of the current tile
+    int turn = __builtin_amdgcn_readfirstlane(cu_slot());
+    take_turn(turn, a.slots);
     for (int it = 0; it < ntiles_k; ++it) {
         const int n0 = it * C::BN;
         const bool more = it + 1 < ntiles_k;
@@ -432,6 +434,7 @@ bwd_dq_kernel(const BwdArgs a) {
             __syncthreads();
         }
         cur = nxt;
+        take_turn(turn, a.slots); // (next to the barrier: the compiler moves nothing across either)
     }
 
     // ---- epilogue: dq = scale * acc rows [0, d), dq_bias = acc rows [16 NKD, 16 NKD + r)
@@ -489,6 +492,8 @@ static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
     const int total = a.ntiles_m * a.B * a.H;
+    static int occupancy = 0;
+    a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, &occupancy);
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
 }

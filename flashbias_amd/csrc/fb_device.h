@@ -396,4 +396,34 @@ __device__ __forceinline__ float half_wave_max(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Turn-taking between the workgroups that share a CU.  The instruction arbiter serves the oldest
+// wave of a SIMD first, so of two resident workgroups the older one runs at the speed it would
+// have alone and the younger one only fills its stalls: their progress differs by a third, and
+// whenever the older one ends the other is left alone with a SIMD it cannot fill.  Raising the
+// wave priority of a different workgroup at every step evens the progress out.  Measured at
+// B2 H4 d32 r8: forward 5 % faster at L = 8192 and 16384, 4 % at 32768; dq kernel 2 % at 16384;
+// the dk/dv kernel (three workgroups per CU, one 32-query step per turn) gained nothing from any
+// rotation tried and does not take turns.
+//
+// cu_slot(): which of the CU's equally sized LDS allocations this workgroup holds (0, 1, ...),
+// read from the LDS_ALLOC hardware register (id 6: base in bits 11:0, size in bits 23:12, same
+// units).  Workgroups of one launch get disjoint allocations at multiples of their size, and a new
+// workgroup inherits the place of the one that ended.  Only a scheduling hint depends on it.
+__device__ __forceinline__ int cu_slot() {
+    const uint32_t r = __builtin_amdgcn_s_getreg((31 << 11) | 6);
+    const uint32_t base = r & 0xfffu, size = (r >> 12) & 0xfffu;
+    return size ? (int)(base / size) : 0;
+}
+
+// Called once per step: the workgroup whose turn it is runs at wave priority 1, the others at 0.
+// `turn` starts as the workgroup's slot and counts round the `nslots` workgroups that share a CU
+// in this launch (wave-uniform values).
+__device__ __forceinline__ void take_turn(int &turn, int nslots) {
+    if (nslots > 1) {
+        if (turn == 0) __builtin_amdgcn_s_setprio(1);
+        else __builtin_amdgcn_s_setprio(0);
+        turn = turn + 1 >= nslots ? 0 : turn + 1;
+    }
+}
+
 } // namespace fb

@@ -332,8 +332,10 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
     if constexpr (C::MTILE) wait_vmcnt<0>();
     __syncthreads();
 
+    int turn = __builtin_amdgcn_readfirstlane(cu_slot());
     for (int it = 0; it < ntiles_k; ++it) {
         const int cur = it & 1;
+        take_turn(turn, a.slots);
         const int n0 = it * C::BN;
         const bool more = it + 1 < ntiles_k;
         if constexpr (C::MTILE) {
@@ -539,6 +541,8 @@ static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
         if (e != hipSuccess) return e;
     }
     const int total = a.ntiles_m * a.B * a.H;
+    static int occupancy = 0;
+    a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, &occupancy);
     hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
     return hipGetLastError();
 }

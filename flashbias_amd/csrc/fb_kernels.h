@@ -16,6 +16,7 @@ struct FwdArgs {
     int causal;
     float scale;
     int ntiles_m; // query tiles per (batch, head)
+    int slots;    // workgroups of this launch that share a compute unit (priority turn-taking)
 };
 
 struct BwdArgs {
@@ -29,6 +30,7 @@ struct BwdArgs {
     float scale;
     int ntiles_n; // key tiles per (batch, head), dk/dv kernel
     int ntiles_m; // query tiles per (batch, head), dq kernel
+    int slots;    // workgroups of this launch that share a compute unit (priority turn-taking)
     int stats_here; // dq kernel: compute -delta and lse * log2(e) itself (and store them) instead of reading them
 };
 
@@ -50,6 +52,21 @@ inline int num_cus() {
         cached[dev] = n; // (idempotent: concurrent first calls store the same value)
     }
     return n;
+}
+
+// Workgroups of a launch of `total` workgroups that sit on one compute unit at a time: what the
+// kernel's registers and LDS admit (queried once per kernel instantiation; *cache holds it), or
+// fewer when the grid does not fill the chip that often.
+template <class K>
+inline int slots_per_cu(K kern, int threads, size_t lds_bytes, int64_t total, int *cache) {
+    int occ = *cache;
+    if (occ == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, threads, lds_bytes) != hipSuccess || occ <= 0) occ = 1;
+        *cache = occ; // (idempotent, as above)
+    }
+    const int64_t cus = num_cus();
+    const int64_t share = (total + cus - 1) / cus;
+    return (int)(share < occ ? (share < 1 ? 1 : share) : occ);
 }
 
 // Padded sizes the dispatchers use: d is covered by 16-wide contraction steps of the
