@@ -14,7 +14,7 @@ FB_MASK_NONE, FB_MASK_VECTOR, FB_MASK_MATRIX = 0, 1, 2
 
 #: every symbol that include/flashbias.h declares
 EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_check", "fb_fwd", "fb_bwd",
-           "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq")
+           "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static")
 
 
 class FbTensor(ctypes.Structure):
@@ -63,7 +63,7 @@ def load():
     lib.fb_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.fb_check.argtypes = [ctypes.POINTER(FbParams), ctypes.c_int]
     lib.fb_check.restype = ctypes.c_int
-    for name in ("fb_fwd", "fb_bwd", "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq"):
+    for name in ("fb_fwd", "fb_bwd", "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static"):
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(FbParams), ctypes.c_void_p]
         fn.restype = ctypes.c_int

@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "flashbias.h"
 #include "fb_kernels.h"
@@ -45,9 +46,40 @@ hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream) {
 }
 } // namespace fb
 
+// Scratch of fb_bwd_static: device memory that belongs to the library image, so that the entry
+// point never calls an allocator.  One copy per GPU that loads the library; it keeps the last
+// call's contents (the backward overwrites every element it later reads, nothing has to start
+// at zero).  In host code the array's name is only a handle for hipGetSymbolAddress: the kernels
+// get the address that call returns.
+static __device__ __align__(256) unsigned char scratch[FB_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char g_err[256] = "";
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {nullptr}; // address of `scratch` on each device, looked up once
+
+// Address of this device's copy of the scratch array (looked up on first use with the device
+// current), or nullptr with *err set.
+void *static_scratch(hipError_t *err) {
+    int dev = 0;
+    *err = hipGetDevice(&dev);
+    if (*err != hipSuccess) return nullptr;
+    if (dev < 0 || dev >= kMaxDevices) {
+        *err = hipErrorInvalidDevice;
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *ptr = nullptr;
+        *err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (*err != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = ptr;
+    }
+    return g_scratch_ptr[dev];
+}
 
 int fail(int code, const char *fmt, const char *what = "") {
     std::snprintf(g_err, sizeof(g_err), fmt, what);
@@ -230,6 +262,24 @@ int fb_bwd_dq(const fb_params *p, void *stream) {
     if (rc) return rc;
     return launched(fb::launch_bwd_dq(bwd_args(p), p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
                     "fb_bwd_dq");
+}
+
+int fb_bwd_static(const fb_params *p, void *stream) {
+    // fb_bwd with the scratch buffer taken from the library's own static device array instead of
+    // fb_params.delta (which is ignored): no allocation, here or in anything it calls.
+    g_err[0] = 0;
+    if (!p) return fail(FB_ERR_NULL, "params: null pointer");
+    if (p->size != sizeof(fb_params)) return fail(FB_ERR_ABI, "fb_params.size does not match this library");
+    const size_t need = fb_bwd_workspace_bytes(p);
+    if (need == 0) return fail(FB_ERR_SHAPE, "B, H, Lq, Lk must be positive");
+    if (need > (size_t)FB_STATIC_SCRATCH_BYTES)
+        return fail(FB_ERR_SHAPE, "fb_bwd_static: B * H * Lq exceeds the static scratch buffer (FB_STATIC_SCRATCH_BYTES); use fb_bwd");
+    hipError_t e = hipSuccess;
+    void *ptr = static_scratch(&e);
+    if (!ptr) return launched(e, "fb_bwd_static (hipGetSymbolAddress)");
+    fb_params q = *p;
+    q.delta = static_cast<float *>(ptr);
+    return fb_bwd(&q, stream);
 }
 
 int fb_bwd(const fb_params *p, void *stream) {

@@ -30,6 +30,9 @@ extern "C" {
 #define FB_VERSION 1
 #define FB_MAX_HEADDIM 128 /* flash_bias_triton.py:1106 */
 #define FB_MAX_RANK 128
+/* Size of the library-owned scratch buffer used by fb_bwd_static (one copy per GPU, held until the
+ * process ends): enough for B * H * Lq <= 4194304 query rows. */
+#define FB_STATIC_SCRATCH_BYTES (32u << 20)
 
 typedef enum fb_status {
     FB_OK = 0,
@@ -110,6 +113,17 @@ int fb_fwd(const fb_params *p, void *stream);
  * registers by a query-stationary kernel and written once, so every gradient is
  * bit-reproducible. */
 int fb_bwd(const fb_params *p, void *stream);
+
+/* fb_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * backward allocates its scratch through torch (flash_bias_triton.py:1212-1219).  Same inputs,
+ * outputs and results as fb_bwd, except that fb_params.delta is ignored: the scratch lives in a
+ * static device array of FB_STATIC_SCRATCH_BYTES inside the library.  Neither this call nor
+ * anything it calls allocates or frees memory.  Returns FB_ERR_SHAPE when
+ * fb_bwd_workspace_bytes(p) exceeds FB_STATIC_SCRATCH_BYTES.  All calls on one GPU share that
+ * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls
+ * ordered on one stream are safe.  Nothing in the array has to be cleared between calls. */
+int fb_bwd_static(const fb_params *p, void *stream);
 
 /* The backward in three phases, exported so that a harness can time them separately (call them in
  * this order: the two main kernels read what the preprocess wrote).

@@ -1,0 +1,58 @@
+"""fb_bwd_static (the backward entry point that allocates nothing) against fb_bwd, through the C ABI."""
+import pytest
+import torch
+
+from _util import make_inputs
+
+
+@pytest.mark.gpu
+def test_static_scratch_backward_matches_fb_bwd(gpu_device):
+    """Two calls in a row, the second on a smaller input: every gradient and nothing else differs
+    from what fb_bwd writes with a caller-owned scratch buffer (bit-exact: same kernels)."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _prepare, _stream, _tensor
+    dev = gpu_device
+    lib = _lib.load()
+
+    def run(B, L, H, d, r, causal, seed):
+        q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=seed)]
+
+        def params(with_scratch):
+            p, keep = _prepare(q, k, v, qb, kb, None, causal, None)
+            bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, L), device=dev, dtype=torch.float32),
+                        dq=torch.full_like(q, float("nan")), dk=torch.full_like(k, float("nan")),
+                        dv=torch.full_like(v, float("nan")),
+                        dqb=torch.full((B, L, H, r), float("nan"), device=dev, dtype=q.dtype),
+                        dkb=torch.full((B, L, H, r), float("nan"), device=dev, dtype=q.dtype))
+            p.o, p.lse, p.dout = _tensor(bufs["o"]), bufs["lse"].data_ptr(), _tensor(do)
+            p.dq, p.dk, p.dv = _tensor(bufs["dq"]), _tensor(bufs["dk"]), _tensor(bufs["dv"])
+            p.dq_bias, p.dk_bias = _tensor(bufs["dqb"]), _tensor(bufs["dkb"])
+            if with_scratch:
+                bufs["scratch"] = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=dev, dtype=torch.float32)
+                p.delta = bufs["scratch"].data_ptr()
+            return p, keep, bufs
+
+        p1, keep1, want = params(True)
+        _lib.check_status(lib.fb_fwd(p1, _stream()))
+        _lib.check_status(lib.fb_bwd(p1, _stream()))
+        p2, keep2, got = params(False)  # delta stays null: the static entry point must not need it
+        _lib.check_status(lib.fb_fwd(p2, _stream()))
+        _lib.check_status(lib.fb_bwd_static(p2, _stream()))
+        torch.cuda.synchronize()
+        for name in ("dq", "dk", "dv", "dqb", "dkb"):
+            assert not torch.isnan(want[name].float()).any(), name
+            assert torch.equal(want[name], got[name]), name
+
+    run(2, 777, 3, 32, 8, True, seed=21)
+    run(1, 130, 2, 32, 8, False, seed=22)  # smaller: the array still holds the first call's values
+
+
+def test_static_scratch_rejects_sizes_beyond_its_array():
+    """The size check comes before anything touches the GPU, so this runs on the CPU."""
+    from flashbias_amd import _lib
+    lib = _lib.load()
+    p = _lib.new_params()
+    p.dtype, p.B, p.H, p.Lq, p.Lk, p.d, p.r, p.scale = _lib.FB_BF16, 64, 64, 2048, 2048, 32, 0, 1.0
+    assert lib.fb_bwd_workspace_bytes(p) > (32 << 20)
+    assert lib.fb_bwd_static(p, None) == -2
+    assert b"static scratch" in lib.fb_last_error()
