@@ -227,9 +227,11 @@ struct FwdLoader {
     }
 };
 
+// The whole forward of one workgroup (C::BM queries of one (batch, head)); the kernel below is
+// nothing else, and the streamlined kernel (fb_fwd_lean.h) calls it for a workgroup whose row sums
+// left the range that its fixed reference point covers.
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU == 1 ? 1 : 2, C::WAVES_EU))) void fwd_kernel(
-    const FwdArgs a) {
+__device__ __forceinline__ void fwd_body(const FwdArgs &a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *sKbuf = reinterpret_cast<uint16_t *>(smem);
     uint16_t *sVbuf = sKbuf + 2 * C::SK_ELEMS;
@@ -529,6 +531,16 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::
     }
 }
 
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU == 1 ? 1 : 2, C::WAVES_EU))) void fwd_kernel(
+    const FwdArgs a) {
+    fwd_body<T, C>(a);
+}
+
+} // namespace fb
+#include "fb_fwd_lean.h"
+namespace fb {
+
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool QB2, bool FOLD>
 static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
     typedef FwdCfg<T, NKD, NKR, NDV, VEC, MASK, QB2, FOLD> C;
@@ -573,6 +585,12 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
     if (a.mask.type)
         return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    if constexpr (NKD <= 2 && NKR <= 1 && NDV == 1) {
+        // the streamlined kernel has 256-query workgroups only: grids that fill the chip (see launch_fwd_vec)
+        const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
+        if (vec && fwd_lean_ok(a) && wgs >= (int64_t)(a.causal ? 7 : 2) * num_cus())
+            return launch_fwd_lean<T, NKD, NKR>(a, stream);
+    }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
     }
