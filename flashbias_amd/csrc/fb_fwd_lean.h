@@ -25,20 +25,31 @@
 //
 // Per score the VALU is left with exp2, the row-sum add and half a convert.
 #pragma once
+#include <type_traits>
 
 namespace fb {
 
-template <class T, int NKD_, int NKR_>
+// LDS layout of one stage (BN keys).  Three regions, each a dense array of 128-byte lines of eight
+// 16-byte chunks: K (64-byte rows, two per line), K_b with a second copy beside it (32-byte rows,
+// four per line), V (64-byte rows).  Row r of a region with CPR chunks per row sits in line
+// r / (8 / CPR) at slot (r % (8 / CPR)) * CPR + chunk, and a slot's position in its line is
+// slot ^ ((line >> 1) & 3): row-wise 16-byte reads of one chunk column by 16 consecutive rows,
+// and the transposing 8-byte reads of V, then touch every bank once.  A copy instruction fills 64
+// consecutive positions (8 lines) of one region, every lane fetching the chunk that belongs at its
+// position: all lanes on, one tensor per instruction, nothing but a scalar base and m0 to set up.
+template <class T, int NKR_>
 struct FwdLeanCfg {
-    static constexpr int NKD = NKD_, NKR = NKR_, NK = NKD_ + NKR_;
-    static_assert(NKD_ <= 2 && NKR_ <= 1, "head dim <= 32, rank <= 8");
-    static constexpr int NWAVES = 4, NTHREADS = 256, BM = 256, BN = 64;
-    static constexpr int ROWCH = 8, ROWCHV = 8; // 128-byte rows of swizzled 16-byte chunks
-    static constexpr int SK = BN * ROWCH * 8, SV = BN * ROWCHV * 8, STAGE = SK + SV;
-    static constexpr int AHEAD = 3, NSTAGE = 4;
-    static constexpr int LDS_BYTES = NSTAGE * STAGE * 2;
+    static constexpr int NKD = 2, NKR = NKR_, NK = NKD + NKR_;
+    static_assert(NKR_ <= 1, "rank <= 8");
+    static constexpr int NWAVES = 4, NTHREADS = 256, BM = 256, BN = 128, KB = BN / 32;
+    static constexpr int K_BYTES = BN * 64, B_BYTES = NKR_ ? BN * 32 : 0, V_BYTES = BN * 64;
+    static constexpr int B_OFF = K_BYTES, V_OFF = K_BYTES + B_BYTES, STAGE_BYTES = V_OFF + V_BYTES;
+    static constexpr int NSTAGE = 3;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
+    // copy instructions per wave and tile: 2 of K (16 rows each), 2 of V, 1 of K_b (32 rows)
+    static constexpr int NDMA = 4 + (NKR_ ? 1 : 0);
     // the general configuration a workgroup falls back to (same 256 queries per workgroup)
-    typedef FwdCfg<T, NKD_, NKR_, 1, true, false, true, false> General;
+    typedef FwdCfg<T, 2, NKR_, 1, true, false, true, false> General;
     static_assert(General::BM == BM && General::LDS_BYTES <= LDS_BYTES, "");
 };
 
@@ -51,11 +62,16 @@ __device__ __attribute__((noinline)) void fwd_lean_retry() {
     fwd_body<T, typename C::General>(a);
 }
 
+// 16 bytes per lane from base + off (base wave-uniform, off a 32-bit byte offset per lane) to LDS
+// byte address lds + 16 * lane; every lane of the wave takes part.
+__device__ __forceinline__ void lds_dma16_all(uint32_t off, const void *base, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "memory");
+}
+
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void fwd_lean_kernel(const FwdArgs a) {
     constexpr int NK = C::NK, NKD = C::NKD, NKR = C::NKR;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-    uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -71,12 +87,13 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int wq0 = m0 + wave * 64; // first query of this wave
 
     const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
-    const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
-    const uint16_t *vbase = a.v.ptr + b * a.v.sb + h * a.v.sh;
-    const uint16_t *qbbase = nullptr, *kbbase = nullptr;
+    const uint8_t *kptr = reinterpret_cast<const uint8_t *>(a.k.ptr + b * a.k.sb + h * a.k.sh);
+    const uint8_t *vptr = reinterpret_cast<const uint8_t *>(a.v.ptr + b * a.v.sb + h * a.v.sh);
+    const uint16_t *qbbase = nullptr;
+    const uint8_t *kbptr = nullptr;
     if constexpr (NKR > 0) {
         qbbase = a.qb.ptr + b * a.qb.sb + h * a.qb.sh;
-        kbbase = a.kb.ptr + b * a.kb.sb + h * a.kb.sh;
+        kbptr = reinterpret_cast<const uint8_t *>(a.kb.ptr + b * a.kb.sb + h * a.kb.sh);
     }
 
     // ---- resident query operands, in exponent-of-2 units (rows past the end are zero)
@@ -96,40 +113,78 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
     const int ntiles_k = (k_end + C::BN - 1) / C::BN;
 
-    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
-        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
-        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
-    }
-    __syncthreads();
-    TileDma<C::BN, C::ROWCH, C::NWAVES, (NKR > 0)> dk;
-    TileDma<C::BN, C::ROWCHV, C::NWAVES, false> dv;
-    constexpr int NDMA = decltype(dk)::NINST + decltype(dv)::NINST; // copy instructions per wave and tile
-    dk.init(kbase, a.k.ss, a.d, 2 * NKD, NKR > 0 ? kbbase : nullptr, NKR > 0 ? a.kb.ss : 0, a.r, wave, lane, 0, true);
-    dv.init(vbase, a.v.ss, a.d, C::ROWCHV, nullptr, 0, 0, wave, lane, 0);
-    auto issue = [&](int stage, int n0) {
-        const uint32_t base = lds_addr_of(stage0 + stage * C::STAGE);
-        dk.issue(base, n0, a.Lk, a.k.ss, NKR > 0 ? a.kb.ss : 0, 2 * NKD);
-        dv.issue(base + 2 * C::SK, n0, a.Lk, a.v.ss, 0, C::ROWCHV);
-    };
-    // Tile t is computed from stage t % 4 and requested three tiles earlier.  When tile t is being
-    // computed, tile t + 1 is already published (the scores of its first block are issued early).
+    // ---- the copies.  This lane's place in an instruction's 8 lines and what belongs there
+    const int dline = lane >> 3, dslot = (lane & 7) ^ ((lane >> 4) & 3);
+    const int krow = 2 * dline + (dslot >> 2), kch = dslot & 3; // K and V regions: row within the 16 rows, chunk
+    const int brow = 4 * dline + (dslot >> 1);                  // K_b region: row within the 32 rows (both chunks: k_b)
+    const int ldk = (int)a.k.ss * 2, ldv = (int)a.v.ss * 2, ldb = NKR > 0 ? (int)a.kb.ss * 2 : 0; // row pitch, bytes
+    // rows [32 wave, 32 wave + 32) of every tile are this wave's to copy
+    uint32_t dk_off[2], dv_off[2], db_off = 0;
 #pragma unroll
-    for (int k = 0; k < C::AHEAD; ++k)
-        if (k < ntiles_k) issue(k, k * C::BN);
-    if (ntiles_k > 2)
-        wait_vmcnt<NDMA>(); // tiles 0 and 1 have landed
+    for (int j = 0; j < 2; ++j) {
+        dk_off[j] = (uint32_t)((32 * wave + 16 * j + krow) * ldk + kch * 16);
+        dv_off[j] = (uint32_t)((32 * wave + 16 * j + krow) * ldv + kch * 16);
+    }
+    if constexpr (NKR > 0) db_off = (uint32_t)((32 * wave + brow) * ldb);
+    const uint32_t lds0 = lds_addr_of(smem);
+    auto issue = [&](int stage, int n0) { // tile n0 .. n0 + BN - 1 into a stage; exactly NDMA copy instructions
+        const uint32_t sb = lds0 + stage * C::STAGE_BYTES + wave * 2048; // (this wave's 16 lines of K and of V)
+        const uint8_t *kt = kptr + (int64_t)n0 * ldk, *vt = vptr + (int64_t)n0 * ldv;
+        if (n0 + C::BN <= a.Lk) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                lds_dma16_all(dk_off[j], kt, sb + j * 1024);
+                lds_dma16_all(dv_off[j], vt, sb + C::V_OFF + j * 1024);
+            }
+            if constexpr (NKR > 0)
+                lds_dma16_all(db_off, kbptr + (int64_t)n0 * ldb, lds0 + stage * C::STAGE_BYTES + C::B_OFF + wave * 1024);
+        } else { // ragged last tile: rows past the end step back to the last key (their scores are hidden)
+            const int last = a.Lk - 1 - n0;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int over = max(32 * wave + 16 * j + krow - last, 0);
+                lds_dma16_all(dk_off[j] - (uint32_t)(over * ldk), kt, sb + j * 1024);
+                lds_dma16_all(dv_off[j] - (uint32_t)(over * ldv), vt, sb + C::V_OFF + j * 1024);
+            }
+            if constexpr (NKR > 0)
+                lds_dma16_all(db_off - (uint32_t)(max(32 * wave + brow - last, 0) * ldb), kbptr + (int64_t)n0 * ldb,
+                              lds0 + stage * C::STAGE_BYTES + C::B_OFF + wave * 1024);
+        }
+    };
+    // Tile t is computed from stage t % 3 and requested two tiles earlier.
+    if (0 < ntiles_k) issue(0, 0);
+    if (1 < ntiles_k) issue(1, C::BN);
+    if (ntiles_k > 1)
+        wait_vmcnt<C::NDMA>(); // tile 0 has landed
     else
         wait_vmcnt<0>();
     __syncthreads();
 
+    // ---- this lane's read addresses inside a stage (stage, key block and step are immediates)
+    uint32_t rk[NKD], rb = 0, rv[2];
+#pragma unroll
+    for (int t = 0; t < NKD; ++t) rk[t] = (c >> 1) * 128 + ((((c & 1) * 4 + 2 * t + g) ^ ((c >> 2) & 3)) * 16);
+    if constexpr (NKR > 0) rb = C::B_OFF + (c >> 2) * 128 + ((((c & 3) * 2 + g) ^ ((c >> 3) & 3)) * 16);
+#pragma unroll
+    for (int hi = 0; hi < 2; ++hi) {
+        const int r = 4 * g + ((c & 15) >> 2) + 8 * hi, chunk = 2 * (c >> 4) + ((c & 3) >> 1);
+        rv[hi] = C::V_OFF + (r >> 1) * 128 + ((((r & 1) * 4 + chunk) ^ ((r >> 2) & 3)) * 16) + 8 * (c & 1);
+    }
     // A operands from LDS: [K | K_b | K_b] rows of key block kb (row-wise), V^T of it (column-wise)
-    auto read_ka = [&](u32x4_t (&f)[NK], const uint16_t *sK, int kb) {
+    auto read_ka = [&](u32x4_t (&f)[NK], int stage, int kb) {
+        const uint8_t *sb = smem + stage * C::STAGE_BYTES;
 #pragma unroll
-        for (int t = 0; t < NK; ++t) f[t] = *reinterpret_cast<const u32x4_t *>(sK + swz_off<C::ROWCH>(kb * 32 + c, 2 * t + g));
+        for (int t = 0; t < NKD; ++t) f[t] = *reinterpret_cast<const u32x4_t *>(sb + rk[t] + kb * 2048);
+        if constexpr (NKR > 0) f[NKD] = *reinterpret_cast<const u32x4_t *>(sb + rb + kb * 1024);
     };
-    auto read_va = [&](u32x4_t (&f)[2], const uint16_t *sK, int kb) {
+    auto read_va = [&](u32x4_t (&f)[2], int stage, int kb) {
+        const uint8_t *sb = smem + stage * C::STAGE_BYTES;
 #pragma unroll
-        for (int t = 0; t < 2; ++t) f[t] = lds_read_a_tr<C::ROWCHV>(sK + C::SK, kb * 32 + 16 * t, 0, c, g);
+        for (int t = 0; t < 2; ++t) {
+            const u32x2_t lo = lds_read_tr4(reinterpret_cast<const uint16_t *>(sb + rv[0] + (kb * 16 + t * 8) * 128));
+            const u32x2_t hi = lds_read_tr4(reinterpret_cast<const uint16_t *>(sb + rv[1] + (kb * 16 + t * 8) * 128));
+            f[t] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+        }
     };
     // exponents of one 32 x 32 block (keys x queries): init + [K | K_b | K_b] [q' | q_b' hi | q_b' lo]^T
     auto scores = [&](const u32x4_t (&f)[NK], int qb, const f32x16_t &init) {
@@ -169,10 +224,28 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         }
     };
 
+    // Instruction order of one block step (LDS reads of the next fragments, the three score MFMAs of
+    // the next block, 40 VALU instructions and the two PV MFMAs of the current one): the independent
+    // score MFMAs go first, spread between the exponentials, so that their results are ready when the
+    // next step starts; then nothing moves across the step boundary.
+    auto interleave = [&]() {
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 16, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
     // ---- reference point of the exponentials: the maximum over the first key block
     u32x4_t ka[NK], kn[NK], va[2];
-    read_ka(ka, stage0, 0);
     {
+        read_ka(ka, 0, 0);
         const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         float mx = -INFINITY;
 #pragma unroll
@@ -190,67 +263,59 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         for (int v = 0; v < 16; ++v) minit[v] = -m2;
     }
 
-    // ---- the key loop: blocks (key block, query block) = (0,0) (0,1) (1,0) (1,1) per tile; s_cur
-    // holds the scores of the tile's first block, issued while the previous tile was finishing
-    f32x16_t s_cur = scores(ka, 0, minit);
-    int cur = 0;
+    // ---- the key loop.  One tile: blocks (key block, query block) = (0,0) (0,1) (1,0) ... (3,1);
+    // the scores of block i + 1 are issued before the exponentials of block i.
     int turn = __builtin_amdgcn_readfirstlane(cu_slot());
-    take_turn(turn, a.slots);
-#pragma unroll 1
-    for (int it = 0; it < ntiles_k; ++it) {
+    auto tile = [&](auto stage_tag, int it) {
+        constexpr int STG = decltype(stage_tag)::value;
         const int n0 = it * C::BN;
-        if (it + C::AHEAD < ntiles_k) issue((cur + C::AHEAD) & 3, n0 + C::AHEAD * C::BN);
-        const uint16_t *sK = stage0 + cur * C::STAGE;
-        const uint16_t *sKn = stage0 + ((cur + 1) & 3) * C::STAGE; // next tile (stale but harmless after the last one)
+        take_turn(turn, a.slots);
+        if (it + 2 < ntiles_k) issue((STG + 2) % 3, n0 + 2 * C::BN);
         const bool edge = n0 + C::BN > a.Lk || (a.causal && n0 + C::BN - 1 > wq0);
-        f32x16_t s_nxt;
+        f32x16_t s_cur, s_nxt;
+        read_ka(ka, STG, 0);
+        s_cur = scores(ka, 0, minit);
+        // one key block: both query blocks against fragments `cur`, the fragments of the next key
+        // block arrive in `nxt` meanwhile
+        auto key_block = [&](u32x4_t (&cur)[NK], u32x4_t (&nxt)[NK], int kb, bool hidden_pairs) {
+            if (kb + 1 < C::KB) read_ka(nxt, STG, kb + 1);
+            read_va(va, STG, kb);
+            s_nxt = scores(cur, 1, minit);
+            if (hidden_pairs) hide(s_cur, n0 + 32 * kb, 0);
+            softmax_pv(s_cur, va, 0);
+            s_cur = s_nxt;
+            interleave();
+            if (kb + 1 < C::KB) s_nxt = scores(nxt, 0, minit);
+            if (hidden_pairs) hide(s_cur, n0 + 32 * kb, 1);
+            softmax_pv(s_cur, va, 1);
+            s_cur = s_nxt;
+            interleave();
+        };
         if (!edge) {
-            read_ka(kn, sK, 1);
-            read_va(va, sK, 0);
-            s_nxt = scores(ka, 1, minit);
-            softmax_pv(s_cur, va, 0);
-            s_cur = s_nxt;
-            s_nxt = scores(kn, 0, minit);
-            softmax_pv(s_cur, va, 1);
-            s_cur = s_nxt;
-            read_ka(ka, sKn, 0);
-            read_va(va, sK, 1);
-            s_nxt = scores(kn, 1, minit);
-            softmax_pv(s_cur, va, 0);
-            s_cur = s_nxt;
-            s_nxt = scores(ka, 0, minit);
-            softmax_pv(s_cur, va, 1);
-            s_cur = s_nxt;
+#pragma unroll
+            for (int kb = 0; kb < C::KB; kb += 2) {
+                key_block(ka, kn, kb, false);
+                key_block(kn, ka, kb + 1, false);
+            }
         } else { // the same with the hidden pairs of every block set to -inf (p = 0)
-            read_ka(kn, sK, 1);
-            read_va(va, sK, 0);
-            s_nxt = scores(ka, 1, minit);
-            hide(s_cur, n0, 0);
-            softmax_pv(s_cur, va, 0);
-            s_cur = s_nxt;
-            s_nxt = scores(kn, 0, minit);
-            hide(s_cur, n0, 1);
-            softmax_pv(s_cur, va, 1);
-            s_cur = s_nxt;
-            read_ka(ka, sKn, 0);
-            read_va(va, sK, 1);
-            s_nxt = scores(kn, 1, minit);
-            hide(s_cur, n0 + 32, 0);
-            softmax_pv(s_cur, va, 0);
-            s_cur = s_nxt;
-            s_nxt = scores(ka, 0, minit);
-            hide(s_cur, n0 + 32, 1);
-            softmax_pv(s_cur, va, 1);
-            s_cur = s_nxt;
+#pragma unroll
+            for (int kb = 0; kb < C::KB; kb += 2) {
+                key_block(ka, kn, kb, true);
+                key_block(kn, ka, kb + 1, true);
+            }
         }
-        // tile it + 2 must have landed before the barrier that lets tile it + 1 start
-        if (it + C::AHEAD < ntiles_k)
-            wait_vmcnt<NDMA>();
+        // the next tile must have landed before the barrier that lets it start
+        if (it + 2 < ntiles_k)
+            wait_vmcnt<C::NDMA>();
         else
             wait_vmcnt<0>();
         barrier_lds();
-        cur = (cur + 1) & 3;
-        take_turn(turn, a.slots);
+    };
+#pragma unroll 1
+    for (int it = 0; it < ntiles_k; it += 3) {
+        tile(std::integral_constant<int, 0>{}, it);
+        if (it + 1 < ntiles_k) tile(std::integral_constant<int, 1>{}, it + 1);
+        if (it + 2 < ntiles_k) tile(std::integral_constant<int, 2>{}, it + 2);
     }
 
     // ---- did every row sum stay in range?  (The decision is the workgroup's: the fallback needs all waves.)
@@ -279,30 +344,29 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
             for (int bq = 0; bq < 4; ++bq) {
                 const int ch = 8 * bq + 4 * g;
-                if (ch + 4 <= a.d) { // (d is a multiple of 8 here)
-                    u32x2_t pk;
-                    pk[0] = T::pack2(acc_o[qb][4 * bq] * inv, acc_o[qb][4 * bq + 1] * inv);
-                    pk[1] = T::pack2(acc_o[qb][4 * bq + 2] * inv, acc_o[qb][4 * bq + 3] * inv);
-                    *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
-                }
+                u32x2_t pk;
+                pk[0] = T::pack2(acc_o[qb][4 * bq] * inv, acc_o[qb][4 * bq + 1] * inv);
+                pk[1] = T::pack2(acc_o[qb][4 * bq + 2] * inv, acc_o[qb][4 * bq + 3] * inv);
+                *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
             }
         }
     }
 }
 
 // Whether the streamlined kernel covers a call (the caller has already checked alignment and the
-// absence of a mask): factors, if any, must fit the hi + lo layout of one bias step.  The bounds
+// absence of a mask): head dim 32 exactly and rank 8 or none (the copies fill whole rows, there is
+// no zero padding of the channels); the factors then fit the hi + lo layout of one bias step.  The bounds
 // on the scale keep the folded operands away from the ends of fp32's range; what a 16-bit type
 // cannot hold after the scaling ends up as inf / NaN row sums, which take the fallback.
 inline bool fwd_lean_ok(const FwdArgs &a) {
     const int64_t lim = (int64_t)1 << 24; // (32-bit tile row offsets in the copies)
-    return a.d <= 32 && a.r <= 8 && a.scale > 1e-6f && a.scale < 1e6f && a.k.ss < lim && a.v.ss < lim &&
+    return a.d == 32 && (a.r == 8 || a.r == 0) && a.scale > 1e-6f && a.scale < 1e6f && a.k.ss < lim && a.v.ss < lim &&
            (a.r == 0 || a.kb.ss < lim);
 }
 
-template <class T, int NKD, int NKR>
+template <class T, int NKR>
 static hipError_t launch_fwd_lean(const FwdArgs &a0, hipStream_t stream) {
-    typedef FwdLeanCfg<T, NKD, NKR> C;
+    typedef FwdLeanCfg<T, NKR> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_lean_kernel<T, C>;
