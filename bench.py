@@ -13,7 +13,17 @@ line:
   cpu_baseline the eager oracle (restated reference eager attention) on the host cores, on a
                bounded sample of the same workload
 
-``--report`` instead prints a table over the other named workloads (not part of the contract).
+The same line carries, beyond the contract's fields: ``gate`` (the tolerance gate of the metric
+evaluated on the very tensors of the timed steps: a subset of query rows against the CPU oracle
+plus the size-independent checksums), ``sweep`` (forward and forward + backward milliseconds of
+every benchmark configuration at its stated size, timed through ``flash_bias_func`` and autograd,
+so that gradient reduction over broadcast factors, rank padding and mask folding are inside),
+``fp16`` (the headline step in fp16, the dtype of the reference's published numbers),
+``factors_permuted_inside`` (the headline step with the (B, H, L, r) -> (B, L, H, r)
+``permute().contiguous()`` of the factors inside the timed region, as flash_bias/benchmark.py:233-235
+times it) and ``providers`` (what PyTorch-ROCm offers for the same math at the headline shape).
+
+``--report`` instead prints a table over more workloads (not part of the contract).
 """
 import argparse
 import json
@@ -26,10 +36,24 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
-# HBM bytes of one dk/dv launch at the headline shape: rocprofv3 FETCH_SIZE (x2.0, calibrated on a copy of
-# known size) + WRITE_SIZE, see profiles/headline_fwd_bwd_kernels.md; a counter figure, not measured live
-DKV_HBM_BYTES = 1.71e8
 PEAK_HBM_GBS = 8000.0
+PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "headline_fwd_bwd_kernels.md")
+
+
+def _profiled_traffic(kernel):
+    """HBM bytes per launch of `kernel` at the headline shape as the tracked rocprofv3 summary states
+    them (a line `hbm_bytes_per_launch <kernel> <bytes>`: FETCH_SIZE and WRITE_SIZE counters scaled
+    by a copy of known size); None when the summary has no such line.  A counter figure, not
+    measured live."""
+    try:
+        with open(PROFILE_SUMMARY) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) >= 3 and parts[0] == "hbm_bytes_per_launch" and parts[1] == kernel:
+                    return float(parts[2])
+    except OSError:
+        pass
+    return None
 
 
 def _to_dev(w, dev):
@@ -121,6 +145,114 @@ def _cpu_baseline(w, flops_per_slice):
             "sample": "%d of B*H (batch, head) slices at full L, one fwd+bwd of the eager oracle in fp32 each" % nslices}
 
 
+def _autograd_ms(leaves, extra, do, steps, warmup, prepare=None):
+    """fwd and fwd+bwd milliseconds of flash_bias_func through autograd (events on the current
+    stream around all the steps).  prepare: work done inside the timed region before the call
+    (returns the factor pair to use)."""
+    import torch
+    from flashbias_amd import flash_bias_func
+    mask, causal, scale = extra
+
+    def fwd():
+        fac = prepare() if prepare else leaves[3:5]
+        return flash_bias_func(leaves[0], leaves[1], leaves[2], fac[0], fac[1], mask, causal, scale)
+
+    def fb():
+        return torch.autograd.grad(fwd(), leaves, do)
+
+    with torch.no_grad():
+        t_fwd = _time_events(fwd, steps, warmup)
+    return t_fwd, _time_events(fb, steps, warmup)
+
+
+def _device_configs(dev):
+    """(name, builder) of every benchmark configuration at its stated size; q, k, v, dO are drawn on
+    the device (timing does not depend on the values), the factors come from the builders."""
+    import torch
+    from flashbias_amd import factors
+
+    def base(B, L, H, d, dtype=torch.bfloat16):
+        return [torch.randn(B, L, H, d, device=dev).to(dtype) for _ in range(4)]
+
+    def sweep(L):
+        q, k, v, do = base(2, L, 4, 32)
+        qb, kb = [(torch.randn(2, L, 4, 8, device=dev) / math.sqrt(8)).bfloat16() for _ in range(2)]
+        return q, k, v, qb, kb, do, False, 8
+
+    def alibi(L):
+        q, k, v, do = base(1, L, 50, 32)
+        qb, kb = factors.alibi_factors(L, L, 50, torch.bfloat16, device=dev)
+        return q, k, v, qb, kb, do, True, 2
+
+    def swin():
+        q, k, v, do = base(4096, 256, 16, 32)
+        qb, kb, _ = factors.svd_factors(factors.swin_v2_bias_table(16, 16, 0), 16, torch.bfloat16)
+        return q, k, v, qb.to(dev), kb.to(dev), do, False, 16
+
+    def pde():
+        q, k, v, do = base(1, 32768, 8, 32)
+        x = torch.rand(1, 32768, 3, device=dev)
+        qb, kb = factors.distance_factors(x, x, 10.0, torch.bfloat16)
+        return q, k, v, qb, kb, do, False, 5
+
+    def pairformer():
+        q, k, v, do = base(768, 768, 4, 32)
+        qb, kb = [(torch.randn(1, 768, 4, 32, device=dev) / math.sqrt(32)).bfloat16() for _ in range(2)]
+        return q, k, v, qb, kb, do, False, 32
+
+    cfgs = [(f"sweep B2 H4 d32 r8 L={L}", lambda L=L: sweep(L)) for L in (1024, 2048, 4096, 8192, 16384)]
+    cfgs += [(f"alibi causal B1 H50 d32 r2 L={L}", lambda L=L: alibi(L)) for L in (2048, 4096, 8192)]
+    cfgs += [("swin 4096 windows x 256 H16 d32 r16 (factors shared by the windows)", swin),
+             ("pde N=32768 H8 d32 r5 (factors shared by the heads)", pde),
+             ("pairformer 768 x 768 H4 d32 r32 (factors shared by the rows)", pairformer)]
+    return cfgs
+
+
+def _sweep(dev, steps, warmup):
+    import torch
+    from flashbias_amd import workloads
+    out = []
+    for name, build in _device_configs(dev):
+        q, k, v, qb, kb, do, causal, r = build()
+        B, L, H, d = q.shape
+        leaves = [t.requires_grad_(True) for t in (q, k, v, qb, kb)]
+        t_fwd, t_fb = _autograd_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
+        f_fwd, f_bwd = workloads.flops(B, H, L, L, d, r, causal)
+        out.append({"workload": name, "fwd_ms": round(t_fwd, 4), "fwd_bwd_ms": round(t_fb, 4),
+                    "fwd_tflops": round(f_fwd / t_fwd / 1e9, 1), "fwd_bwd_tflops": round((f_fwd + f_bwd) / t_fb / 1e9, 1),
+                    "pct_of_bf16_mfma_peak": round(100 * (f_fwd + f_bwd) / t_fb / 1e9 / PEAK_BF16_TFLOPS, 2)})
+        del q, k, v, qb, kb, do, leaves
+        torch.cuda.empty_cache()
+    return out
+
+
+def _gate(w, o, grads):
+    """The tolerance gate of the metric on the tensors of a timed step: o, dq, dq_bias of 192 query
+    rows against the CPU oracle run on (those rows, all keys); dk, dv, dk_bias through the
+    identities sum_j dv_j = sum_i dO_i and sum_j dk_j = 0 = sum_j dk_bias_j."""
+    import torch
+    from oracle import eager
+    L = w["q"].shape[1]
+    rows = torch.cat([torch.arange(0, 64), torch.arange(L // 2 - 32, L // 2 + 32), torch.arange(L - 64, L)])
+    f = lambda t: t.detach().float().cpu()
+    sub = lambda t: f(t[:, rows])
+    ref = eager.flashbias_eager_grads(sub(w["q"]), f(w["k"]), f(w["v"]), sub(w["q_bias"]), f(w["k_bias"]), None, False,
+                                      w["softmax_scale"], sub(w["do"]))
+    rel = lambda got, want: ((f(got) - want).abs().max() / want.abs().max()).item()
+    o_err = (f(o[:, rows]) - ref[0]).abs().max().item()
+    ratios = {"dq": rel(grads[0][:, rows], ref[1]), "dq_bias": rel(grads[3][:, rows], ref[4])}
+    do_sum = w["do"].float().sum(1)
+    ratios["dv (column sums)"] = ((grads[2].float().sum(1) - do_sum).abs().max() / do_sum.abs().max()).item()
+    for name, gk in (("dk (column sums)", grads[1]), ("dk_bias (column sums)", grads[4])):
+        gk = gk.float()
+        ratios[name] = (gk.sum(1).abs().max() / (gk.abs().sum(1).max() / math.sqrt(gk.shape[1]))).item()
+    ok = (o_err <= 2e-2 and ratios["dq"] <= 5e-2 and ratios["dq_bias"] <= 5e-2 and ratios["dv (column sums)"] <= 2e-2
+          and ratios["dk (column sums)"] <= 16 * 2.0 ** -9 and ratios["dk_bias (column sums)"] <= 16 * 2.0 ** -9)
+    return {"pass": bool(ok), "o_max_abs_err": round(o_err, 5), "o_tol": 2e-2, "grad_tol": 5e-2,
+            "ratios": {k: round(v, 5) for k, v in ratios.items()},
+            "checked": "192 query rows x all keys of o, dq, dq_bias against the fp32 CPU oracle; column sums of dv, dk, dk_bias"}
+
+
 def headline(args):
     import torch
     from flashbias_amd import flash_bias_func, workloads
@@ -131,16 +263,18 @@ def headline(args):
 
     def step():
         o = flash_bias_func(*leaves, None, False, w["softmax_scale"])
-        return torch.autograd.grad(o, leaves, w["do"])
+        return o, torch.autograd.grad(o, leaves, w["do"])
 
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        last = step()
     torch.cuda.synchronize()
     ms_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    gate = _gate(w, last[0].detach(), last[1])
+    del last
 
     f_fwd, f_bwd = workloads.flops(hl["B"], hl["H"], hl["L"], hl["L"], hl["d"], hl["r"])
     phases, keep = _phase_timers({n: (t.detach() if isinstance(t, torch.Tensor) else t) for n, t in w.items()}, dev)
@@ -175,9 +309,37 @@ def headline(args):
         "reference_formula_tflops": round(ref_fb / (ms_step * 1e-3) / 1e12, 2),
         "roofline": {"kernel": "bwd_dkv_kernel (fb_bwd_dkv)", "bound": "mfma", "achieved": round(tflops_main, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_main / PEAK_BF16_TFLOPS, 4),
-                     "traffic": DKV_HBM_BYTES},
+                     "traffic": _profiled_traffic("bwd_dkv_kernel")},
+        "gate": gate,
     }
     del keep
+    if not args.no_extras:
+        steps, warm = max(5, args.steps // 2), max(2, args.warmup // 2)
+        extra = (None, False, w["softmax_scale"])
+        # the factors as flash_bias/benchmark.py:220-235 creates them, permuted inside the timed step
+        stored = [w[n].detach().permute(0, 2, 1, 3).contiguous() for n in ("q_bias", "k_bias")]  # (B, H, L, r)
+        fac_leaves = leaves[:3] + [t.requires_grad_(True) for t in stored]
+        inside = _autograd_ms(fac_leaves, extra, w["do"], steps, warm,
+                              prepare=lambda: [t.permute(0, 2, 1, 3).contiguous() for t in fac_leaves[3:]])
+        out["factors_permuted_inside"] = {"fwd_ms": round(inside[0], 4), "fwd_bwd_ms": round(inside[1], 4)}
+        del stored, fac_leaves
+        half = [w[n].detach().half().requires_grad_(True) for n in ("q", "k", "v", "q_bias", "k_bias")]
+        t16 = _autograd_ms(half, extra, w["do"].half(), steps, warm)
+        out["fp16"] = {"fwd_ms": round(t16[0], 4), "fwd_bwd_ms": round(t16[1], 4),
+                       "fwd_bwd_tflops": round((f_fwd + f_bwd) / t16[1] / 1e9, 1),
+                       "pct_of_fp16_mfma_peak": round(100 * (f_fwd + f_bwd) / t16[1] / 1e9 / PEAK_BF16_TFLOPS, 2)}
+        del half
+        cat = _time_torch(lambda: _sdpa_concat(w), leaves, w["do"], 3, 1)
+        with torch.no_grad():
+            bias = (w["q_bias"].permute(0, 2, 1, 3) @ w["k_bias"].permute(0, 2, 3, 1)).contiguous()
+        den = _time_torch(lambda: _sdpa_dense(w, bias), leaves[:3], w["do"], 3, 1)
+        del bias
+        out["providers"] = {"torch SDPA on concatenated [q*scale, q_bias] / [k, k_bias] (attention_func.py:188-237)":
+                            {"fwd_ms": round(cat[0], 3), "fwd_bwd_ms": round(cat[1], 3)},
+                            "torch SDPA with the materialised dense bias (attention_func.py:150-185; no factor gradients)":
+                            {"fwd_ms": round(den[0], 3), "fwd_bwd_ms": round(den[1], 3)}}
+        torch.cuda.empty_cache()
+        out["sweep"] = _sweep(dev, steps, warm)
     if not args.no_cpu:
         out["cpu_baseline"] = _cpu_baseline(w, (f_fwd + f_bwd) / (hl["B"] * hl["H"]))
     print(json.dumps(out))
@@ -274,6 +436,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the sweep, fp16, permuted-factors and provider timings (profiling runs)")
     ap.add_argument("--report", action="store_true", help="table over all named workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the run, copy a 256 MiB buffer 3 times (a plain copy kernel of known size, "

@@ -16,16 +16,44 @@ def alibi_slopes(nheads):
     return torch.pow(2.0, -8.0 * h / nheads).float()
 
 
-def alibi_factors(seqlen_q, seqlen_k, nheads, dtype=torch.float32, device=None):
-    """Exact rank-2 factors of the ALiBi bias  -m_h (i - j):
-    q_bias[i] = [-m_h i, 1],  k_bias[j] = [1, m_h j].
-    (The demo module of the reference, attention_with_alibi_bias.py:49-52, uses the opposite
-    sign; this is the standard ALiBi penalty.)  Computed in fp32, cast once."""
+def alibi_factors(seqlen_q, seqlen_k, nheads, dtype=torch.float32, device=None, exact=False, reference_sign=False):
+    """Factors of the ALiBi bias  -m_h (i - j)  (``reference_sign``: +m_h (i - j), what the
+    reference's demo module builds, 1_Language_Model/attention_with_alibi_bias.py:49-52).
+
+    ``exact=False``: the rank-2 closed form  q_bias[i] = [-m_h i, 1],  k_bias[j] = [1, m_h j],
+    computed in fp32 and cast once.  In a 16-bit dtype the columns m_h i are rounded to 8 (bf16)
+    or 11 (fp16) significant bits, so the product of the cast factors deviates from the closed
+    form by up to several units at positions in the thousands.
+
+    ``exact=True``: rank-4 factors whose every column is exactly representable in bf16 and fp16
+    for positions below 65536, with i = 256 a_i + b_i and the slope rounded to the dtype once:
+
+        q_bias[i] = [a_i, b_i, 256 m, m],   k_bias[j] = [-256 m, -m, a_j, b_j]
+
+    The four products and their fp32 sum are exact, so the kernels see exactly  -m (i - j)  with
+    m = the 16-bit slope: monotone in the distance, relative deviation from the true slope at most
+    half an ulp of the dtype.  This is what the module drop-in uses."""
     m = alibi_slopes(nheads).to(device)
-    i = torch.arange(seqlen_q, dtype=torch.float32, device=device)
-    j = torch.arange(seqlen_k, dtype=torch.float32, device=device)
-    q_bias = torch.stack([-(i[:, None] * m[None, :]), torch.ones(seqlen_q, nheads, device=device)], dim=-1)
-    k_bias = torch.stack([torch.ones(seqlen_k, nheads, device=device), j[:, None] * m[None, :]], dim=-1)
+    if not exact:
+        i = torch.arange(seqlen_q, dtype=torch.float32, device=device)
+        j = torch.arange(seqlen_k, dtype=torch.float32, device=device)
+        sgn = 1.0 if reference_sign else -1.0
+        q_bias = torch.stack([sgn * (i[:, None] * m[None, :]), torch.ones(seqlen_q, nheads, device=device)], dim=-1)
+        k_bias = torch.stack([torch.ones(seqlen_k, nheads, device=device), -sgn * (j[:, None] * m[None, :])], dim=-1)
+        return q_bias[None].to(dtype), k_bias[None].to(dtype)
+    assert max(seqlen_q, seqlen_k) <= 65536, "positions are split into two 8-bit digits"
+    m = m.to(dtype).float()  # the slope the kernels will see
+    sgn = -1.0 if reference_sign else 1.0
+
+    def digits(n):
+        pos = torch.arange(n, device=device)
+        return (pos // 256).float()[:, None].expand(n, nheads), (pos % 256).float()[:, None].expand(n, nheads)
+
+    aq, bq = digits(seqlen_q)
+    ak, bk = digits(seqlen_k)
+    mq, mk = m[None, :].expand(seqlen_q, nheads), m[None, :].expand(seqlen_k, nheads)
+    q_bias = torch.stack([aq, bq, 256.0 * mq, mq], dim=-1)
+    k_bias = torch.stack([-sgn * 256.0 * mk, -sgn * mk, sgn * ak, sgn * bk], dim=-1)
     return q_bias[None].to(dtype), k_bias[None].to(dtype)
 
 

@@ -91,8 +91,14 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
         assert k_bias.shape[-1] == rank
         if rank % 8:
             # zero columns change nothing in q_bias k_bias^T; a multiple of 8 makes the rows 16-byte
-            # aligned, which selects the kernels with vector loads (ALiBi r=2, distance bias r=5)
-            pad = (0, 8 - rank % 8)
+            # aligned, which selects the kernels with vector loads (ALiBi r=2, distance bias r=5).
+            # Ranks below 8 are padded to 16, not 8: they are closed-form factors whose columns can be
+            # large functions of position (ALiBi: m * i in the thousands, cancelling against m * j),
+            # and a rank of 16 selects the kernels that keep the factors as they are and apply the
+            # softmax scale to the fp32 accumulator.  The kernels that fold the scale into a 16-bit
+            # operand (rank 8) carry every bias term with a relative error of 2^-17, which is 0.05 in
+            # the logits at |term| = 7000.
+            pad = (0, (16 if rank < 8 else -(-rank // 8) * 8) - rank)
             q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
             rank = q_bias.shape[-1]
         # (padding a permuted view keeps its permuted layout)

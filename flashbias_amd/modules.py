@@ -15,11 +15,16 @@ class AttentionWithALiBiBias(nn.Module):
     """Causal multi-head self-attention with ALiBi as an exact rank-2 FlashBias.
 
     Same constructor arguments and forward contract as the reference module
-    (x: (batch, seq, dim) -> (batch, seq, dim)); the bias factors follow the standard ALiBi sign,
-    ``-m_h (i - j)`` (``factors.alibi_factors``)."""
+    (x: (batch, seq, dim) -> (batch, seq, dim)).  Two deliberate differences, both switchable:
+    the bias follows the standard ALiBi sign, ``-m_h (i - j)``, unless ``reference_sign=True``
+    (the reference builds ``+m_h (i - j)``, attention_with_alibi_bias.py:49-52), and the compute
+    dtype defaults to bf16 where the reference casts to fp16 (``dtype=torch.float16`` restores
+    that).  The factors are the exact rank-4 form of ``factors.alibi_factors``: the bias the
+    kernels see is exactly ``-m (i - j)`` with the slope rounded to the dtype, at every position."""
 
-    def __init__(self, dim, heads, dim_head, dropout=0.0, dtype=torch.bfloat16):
+    def __init__(self, dim, heads, dim_head, dropout=0.0, dtype=torch.bfloat16, reference_sign=False):
         super().__init__()
+        self.reference_sign = reference_sign
         inner = dim_head * heads
         self.heads, self.dim_head, self.scale, self.dtype = heads, dim_head, dim_head ** -0.5, dtype
         self.to_q = nn.Linear(dim, inner, bias=False)
@@ -31,7 +36,8 @@ class AttentionWithALiBiBias(nn.Module):
         b, n, _ = x.shape
         split = lambda t: t.view(b, n, self.heads, self.dim_head).to(self.dtype)
         q, k, v = split(self.to_q(x)), split(self.to_k(x)), split(self.to_v(x))
-        q_bias, k_bias = factors.alibi_factors(n, n, self.heads, self.dtype, x.device)
+        q_bias, k_bias = factors.alibi_factors(n, n, self.heads, self.dtype, x.device, exact=True,
+                                               reference_sign=self.reference_sign)
         o = flash_bias_func(q, k, v, q_bias, k_bias, None, True, self.scale)
         return self.to_out(o.reshape(b, n, -1).to(x.dtype))
 

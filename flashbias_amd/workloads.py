@@ -52,11 +52,13 @@ def plumbing(seed=0):
     return sweep(1024, dtype=torch.float32, seed=seed)
 
 
-def alibi(L, H=50, d=32, dtype=torch.bfloat16, seed=0):
-    """Causal LM with ALiBi as an exact rank-2 bias, B1 H50 d32."""
+def alibi(L, H=50, d=32, dtype=torch.bfloat16, seed=0, exact=False):
+    """Causal LM with ALiBi as a rank-2 bias, B1 H50 d32: q_bias[i] = [-m_h i, 1], k_bias[j] =
+    [1, m_h j], computed in fp32 and cast (the checker consumes the cast factors).  exact=True: the
+    rank-4 factors that are exact in 16 bits (factors.alibi_factors)."""
     g = torch.Generator().manual_seed(seed)
     q, k, v, do = _qkv(1, L, L, H, d, g, dtype)
-    qb, kb = factors.alibi_factors(L, L, H, dtype)
+    qb, kb = factors.alibi_factors(L, L, H, dtype, exact=exact)
     return _pack(q, k, v, do, qb, kb, True, 1.0 / math.sqrt(d))
 
 

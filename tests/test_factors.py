@@ -25,6 +25,33 @@ def test_alibi_slopes_and_factors_closed_form():
     assert torch.allclose(_dense(qb, kb)[0], want, atol=1e-5)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("reference_sign", [False, True])
+def test_alibi_factors_exact_in_16_bits(dtype, reference_sign):
+    """The rank-4 factors: the product of the 16-bit factors equals -m (i - j) exactly, with m the
+    slope rounded to the dtype, at positions up to 8192 and beyond; the rank-2 closed form cast
+    to 16 bits is off by units there (which is why the module does not use it)."""
+    H, L = 8, 8192 + 300
+    qb, kb = factors.alibi_factors(L, L, H, dtype, exact=True, reference_sign=reference_sign)
+    assert qb.shape == (1, L, H, 4) and kb.shape == (1, L, H, 4) and qb.dtype == dtype
+    m = factors.alibi_slopes(H).to(dtype).double()
+    rows = torch.tensor([0, 1, 255, 256, 257, 1000, 4095, 4096, 8191, 8192, L - 1])
+    got = torch.einsum("ihr,jhr->hij", qb[0, rows].double(), kb[0].double())
+    sgn = 1.0 if reference_sign else -1.0
+    want = sgn * m[:, None, None] * (rows.double()[None, :, None] - torch.arange(L).double()[None, None, :])
+    assert torch.equal(got, want)
+    # and in fp32 accumulation, which is what the kernels do
+    got32 = torch.einsum("ihr,jhr->hij", qb[0, rows].float(), kb[0].float())
+    assert torch.equal(got32.double(), want)
+    true = sgn * factors.alibi_slopes(H).double()[:, None, None] * (rows.double()[None, :, None] - torch.arange(L).double()[None, None, :])
+    ulp = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert ((got - true).abs() <= ulp * true.abs() + 1e-12).all()
+    # the cast rank-2 form, for comparison
+    q2, k2 = factors.alibi_factors(L, L, H, dtype, reference_sign=reference_sign)
+    err2 = (torch.einsum("ihr,jhr->hij", q2[0, rows].double(), k2[0].double()) - true).abs().max()
+    assert err2 > 0.4
+
+
 def test_distance_factors_identity():
     """-alpha |x_i - x_j|^2 = [-alpha|x_i|^2, -alpha, 2 alpha x_i] . [1, |x_j|^2, x_j], exact rank D+2."""
     g = torch.Generator().manual_seed(0)
