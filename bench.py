@@ -93,10 +93,10 @@ def _phase_timers(w, dev):
     (buffers allocated once, outside the timed region)."""
     import torch
     from flashbias_amd import _lib
-    from flashbias_amd.interface import _prepare, _stream, _tensor
+    from flashbias_amd.interface import _params, _stream, _tensor
     lib = _lib.load()
     q, k, v, qb, kb, do = (w[n] for n in ("q", "k", "v", "q_bias", "k_bias", "do"))
-    p, keep = _prepare(q, k, v, qb, kb, w.get("mask"), w["causal"], w["softmax_scale"])
+    p, keep = _params(q, k, v, qb, kb, w.get("mask"), w["causal"], w["softmax_scale"])
     o = torch.empty_like(q)
     lse = torch.empty((p.B, p.H, p.Lq), device=dev, dtype=torch.float32)
     p.o, p.lse = _tensor(o), lse.data_ptr()

@@ -1,12 +1,13 @@
-// C ABI of the library (declared in include/flashbias.h): argument checks that run without
-// a GPU, translation of fb_params into kernel argument blocks, dispatch to the instantiation
-// that covers (dtype, head dim, rank).
+// C ABI of the library (declared in include/flashbias.h): translation of fb_params into kernel
+// argument blocks and dispatch to the instantiation that covers (dtype, head dim, rank).  The
+// argument checks themselves (fb_check) are plain C++ in fb_checks.cpp.
 #include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
 
 #include "flashbias.h"
+#include "fb_checks.h"
 #include "fb_kernels.h"
 
 namespace fb {
@@ -55,8 +56,6 @@ static __device__ __align__(256) unsigned char scratch[FB_STATIC_SCRATCH_BYTES];
 
 namespace {
 
-thread_local char g_err[256] = "";
-
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void *g_scratch_ptr[kMaxDevices] = {nullptr}; // address of `scratch` on each device, looked up once
@@ -79,11 +78,6 @@ void *static_scratch(hipError_t *err) {
         g_scratch_ptr[dev] = ptr;
     }
     return g_scratch_ptr[dev];
-}
-
-int fail(int code, const char *fmt, const char *what = "") {
-    std::snprintf(g_err, sizeof(g_err), fmt, what);
-    return code;
 }
 
 bool vec_ok(const fb_tensor &t) {
@@ -113,23 +107,6 @@ fb::MaskDesc dev_mask(const fb_params *p) {
     m.vec_ok = p->mask_type && reinterpret_cast<uintptr_t>(m.ptr) % align == 0 && m.sb % 4 == 0 && m.sh % 4 == 0 &&
                m.sm % 4 == 0;
     return m;
-}
-
-// input: may broadcast over batch / head (stride 0), never negative strides
-int check_in(const fb_tensor &t, int channels, const char *name) {
-    if (!t.ptr) return fail(FB_ERR_NULL, "%s: null pointer", name);
-    if (t.stride_b < 0 || t.stride_h < 0 || t.stride_s < 0) return fail(FB_ERR_STRIDE, "%s: negative stride", name);
-    (void)channels;
-    return FB_OK;
-}
-
-// output: rows must not alias each other
-int check_out(const fb_tensor &t, int channels, int B, int H, int L, const char *name) {
-    if (!t.ptr) return fail(FB_ERR_NULL, "%s: null pointer", name);
-    if (t.stride_b < 0 || t.stride_h < 0 || t.stride_s < 0) return fail(FB_ERR_STRIDE, "%s: negative stride", name);
-    if ((L > 1 && t.stride_s < channels) || (B > 1 && t.stride_b == 0) || (H > 1 && t.stride_h == 0))
-        return fail(FB_ERR_STRIDE, "%s: output rows alias (zero or too small stride)", name);
-    return FB_OK;
 }
 
 fb::FwdArgs fwd_args(const fb_params *p) {
@@ -179,63 +156,12 @@ fb::BwdArgs bwd_args(const fb_params *p) {
 
 int launched(hipError_t e, const char *what) {
     if (e == hipSuccess) return FB_OK;
-    std::snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString(e));
-    return FB_ERR_LAUNCH;
+    return fb::api_fail(FB_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
 }
 
 } // namespace
 
 extern "C" {
-
-int fb_version(void) { return FB_VERSION; }
-
-const char *fb_last_error(void) { return g_err; }
-
-size_t fb_bwd_workspace_bytes(const fb_params *p) {
-    if (!p || p->B <= 0 || p->H <= 0 || p->Lq <= 0) return 0;
-    return (size_t)2 * (size_t)p->B * (size_t)p->H * (size_t)p->Lq * sizeof(float);
-}
-
-int fb_check(const fb_params *p, int pass) {
-    g_err[0] = 0;
-    if (!p) return fail(FB_ERR_NULL, "params: null pointer");
-    if (p->size != sizeof(fb_params)) return fail(FB_ERR_ABI, "fb_params.size does not match this library");
-    if (p->dtype != FB_F16 && p->dtype != FB_BF16) return fail(FB_ERR_DTYPE, "only fp16 and bf16 are supported");
-    if (p->B <= 0 || p->H <= 0 || p->Lq <= 0 || p->Lk <= 0) return fail(FB_ERR_SHAPE, "B, H, Lq, Lk must be positive");
-    if (p->d <= 0 || p->d > FB_MAX_HEADDIM) return fail(FB_ERR_SHAPE, "head dim must be in 1..128");
-    if (p->r < 0 || p->r > FB_MAX_RANK) return fail(FB_ERR_SHAPE, "bias rank must be in 0..128");
-    if (!std::isfinite(p->scale) || p->scale == 0.f) return fail(FB_ERR_SCALE, "softmax scale must be finite and non-zero");
-    int rc;
-    if ((rc = check_in(p->q, p->d, "q"))) return rc;
-    if ((rc = check_in(p->k, p->d, "k"))) return rc;
-    if ((rc = check_in(p->v, p->d, "v"))) return rc;
-    if (p->r > 0) {
-        if ((rc = check_in(p->q_bias, p->r, "q_bias"))) return rc;
-        if ((rc = check_in(p->k_bias, p->r, "k_bias"))) return rc;
-    }
-    if (p->mask_type != FB_MASK_NONE) {
-        if (p->mask_type != FB_MASK_VECTOR && p->mask_type != FB_MASK_MATRIX)
-            return fail(FB_ERR_MASK, "mask_type must be none, vector or matrix");
-        if (p->mask_dtype != p->dtype && p->mask_dtype != FB_F32)
-            return fail(FB_ERR_MASK, "mask must have the input dtype or fp32");
-        if (!p->mask.ptr) return fail(FB_ERR_NULL, "%s: null pointer", "mask");
-        if (p->mask.stride_b < 0 || p->mask.stride_h < 0 || p->mask.stride_s < 0)
-            return fail(FB_ERR_STRIDE, "%s: negative stride", "mask");
-    }
-    if (!p->lse) return fail(FB_ERR_NULL, "%s: null pointer", "lse");
-    if (pass == 0) return check_out(p->o, p->d, p->B, p->H, p->Lq, "o");
-    if ((rc = check_in(p->o, p->d, "o"))) return rc;
-    if ((rc = check_in(p->dout, p->d, "dout"))) return rc;
-    if ((rc = check_out(p->dq, p->d, p->B, p->H, p->Lq, "dq"))) return rc;
-    if ((rc = check_out(p->dk, p->d, p->B, p->H, p->Lk, "dk"))) return rc;
-    if ((rc = check_out(p->dv, p->d, p->B, p->H, p->Lk, "dv"))) return rc;
-    if (p->r > 0) {
-        if ((rc = check_out(p->dq_bias, p->r, p->B, p->H, p->Lq, "dq_bias"))) return rc;
-        if ((rc = check_out(p->dk_bias, p->r, p->B, p->H, p->Lk, "dk_bias"))) return rc;
-    }
-    if (!p->delta) return fail(FB_ERR_NULL, "%s: null pointer", "delta");
-    return FB_OK;
-}
 
 int fb_fwd(const fb_params *p, void *stream) {
     const int rc = fb_check(p, 0);
@@ -267,13 +193,13 @@ int fb_bwd_dq(const fb_params *p, void *stream) {
 int fb_bwd_static(const fb_params *p, void *stream) {
     // fb_bwd with the scratch buffer taken from the library's own static device array instead of
     // fb_params.delta (which is ignored): no allocation, here or in anything it calls.
-    g_err[0] = 0;
-    if (!p) return fail(FB_ERR_NULL, "params: null pointer");
-    if (p->size != sizeof(fb_params)) return fail(FB_ERR_ABI, "fb_params.size does not match this library");
+    fb::api_clear_error();
+    if (!p) return fb::api_fail(FB_ERR_NULL, "params: null pointer");
+    if (p->size != sizeof(fb_params)) return fb::api_fail(FB_ERR_ABI, "fb_params.size does not match this library");
     const size_t need = fb_bwd_workspace_bytes(p);
-    if (need == 0) return fail(FB_ERR_SHAPE, "B, H, Lq, Lk must be positive");
+    if (need == 0) return fb::api_fail(FB_ERR_SHAPE, "B, H, Lq, Lk must be positive");
     if (need > (size_t)FB_STATIC_SCRATCH_BYTES)
-        return fail(FB_ERR_SHAPE, "fb_bwd_static: B * H * Lq exceeds the static scratch buffer (FB_STATIC_SCRATCH_BYTES); use fb_bwd");
+        return fb::api_fail(FB_ERR_SHAPE, "fb_bwd_static: B * H * Lq exceeds the static scratch buffer (FB_STATIC_SCRATCH_BYTES); use fb_bwd");
     hipError_t e = hipSuccess;
     void *ptr = static_scratch(&e);
     if (!ptr) return launched(e, "fb_bwd_static (hipGetSymbolAddress)");

@@ -114,6 +114,7 @@ static void launch_preprocess_t(const BwdArgs &a, hipStream_t stream) {
 }
 
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream) {
+    (void)hipGetLastError(); // (an earlier, unrelated error of the process is not this launch's)
     if (bf16)
         launch_preprocess_t<BF16>(a, stream);
     else

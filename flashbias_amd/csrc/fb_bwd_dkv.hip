@@ -561,14 +561,10 @@ static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
     BwdArgs a = a0;
     a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
     auto kern = bwd_dkv_kernel<T, C>;
-    if (C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-        if (e != hipSuccess) return e;
-    }
-    const int total = a.ntiles_n * a.B * a.H;
-    hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
-    return hipGetLastError();
+    static KernelOnce once;
+    const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
+    if (e != hipSuccess) return e;
+    return launch_flat(kern, (int64_t)a.ntiles_n * a.B * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
 }
 
 // One pass, or (head dims above 64, aligned tensors) two or three passes that each keep a part

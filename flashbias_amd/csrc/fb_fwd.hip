@@ -547,16 +547,12 @@ static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_kernel<T, C>;
-    if (C::LDS_BYTES > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
-        if (e != hipSuccess) return e;
-    }
-    const int total = a.ntiles_m * a.B * a.H;
-    static int occupancy = 0;
-    a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, &occupancy);
-    hipLaunchKernelGGL(kern, dim3(total), dim3(C::NTHREADS), C::LDS_BYTES, stream, a);
-    return hipGetLastError();
+    static KernelOnce once;
+    const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
+    if (e != hipSuccess) return e;
+    const int64_t total = (int64_t)a.ntiles_m * a.B * a.H;
+    a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, once);
+    return launch_flat(kern, total, C::NTHREADS, C::LDS_BYTES, stream, a);
 }
 
 // Two query blocks per wave (256 queries per workgroup) pay once every compute unit has two such

@@ -1,5 +1,6 @@
 // Host-visible kernel argument blocks and launchers (implemented in fb_fwd.hip / fb_bwd.hip).
 #pragma once
+#include <atomic>
 #include <cmath>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -43,26 +44,54 @@ hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream);
 // Compute units of the current device (cached per device; 256 on MI355X).  The launchers pick
 // smaller query tiles when the larger ones would leave compute units without a workgroup.
 inline int num_cus() {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
-    int n = cached[dev];
+    int n = cached[dev].load(std::memory_order_relaxed);
     if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-        cached[dev] = n; // (idempotent: concurrent first calls store the same value)
+        cached[dev].store(n, std::memory_order_relaxed); // (concurrent first calls store the same value)
     }
     return n;
+}
+
+// What a launcher remembers about one kernel instantiation (one static object per instantiation;
+// the only mutable state of the library besides num_cus() and fb_bwd_static's scratch address:
+// write-once values, atomics, so concurrent first calls from several threads are fine).
+struct KernelOnce {
+    std::atomic<int> lds_set{0};   // the dynamic-LDS limit of the kernel has been raised
+    std::atomic<int> occupancy{0}; // workgroups per compute unit that registers and LDS admit
+};
+
+// Raises the kernel's dynamic LDS limit on its first launch if it needs more than the default 48 KB.
+template <class K>
+inline hipError_t allow_lds(K kern, size_t lds_bytes, KernelOnce &once) {
+    if (lds_bytes <= 48 * 1024 || once.lds_set.load(std::memory_order_acquire)) return hipSuccess;
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (int)lds_bytes);
+    if (e == hipSuccess) once.lds_set.store(1, std::memory_order_release);
+    return e;
+}
+
+// One-dimensional launch; the error it returns is this launch's own (an error that some earlier,
+// unrelated call of the process left behind is cleared first, not reported as ours).
+template <class K, class A>
+inline hipError_t launch_flat(K kern, int64_t total, int threads, size_t lds_bytes, hipStream_t stream, const A &args) {
+    if (total <= 0 || total > 0x7fffffffLL) return hipErrorInvalidConfiguration; // (fb_check bounds the sizes)
+    (void)hipGetLastError();
+    hipLaunchKernelGGL(kern, dim3((unsigned)total), dim3(threads), lds_bytes, stream, args);
+    return hipGetLastError();
 }
 
 // Workgroups of a launch of `total` workgroups that sit on one compute unit at a time: what the
 // kernel's registers and LDS admit (queried once per kernel instantiation; *cache holds it), or
 // fewer when the grid does not fill the chip that often.
 template <class K>
-inline int slots_per_cu(K kern, int threads, size_t lds_bytes, int64_t total, int *cache) {
-    int occ = *cache;
+inline int slots_per_cu(K kern, int threads, size_t lds_bytes, int64_t total, KernelOnce &once) {
+    int occ = once.occupancy.load(std::memory_order_relaxed);
     if (occ == 0) {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kern, threads, lds_bytes) != hipSuccess || occ <= 0) occ = 1;
-        *cache = occ; // (idempotent, as above)
+        once.occupancy.store(occ, std::memory_order_relaxed); // (concurrent first calls store the same value)
     }
     const int64_t cus = num_cus();
     const int64_t share = (total + cus - 1) / cus;

@@ -1,0 +1,57 @@
+// Sanitizer driver for the argument checks and size queries of the C ABI (fb_checks.cpp), built
+// under AddressSanitizer and UBSan by `make sanitize` and called with well-formed and with
+// deliberately malformed parameter blocks.  No GPU is involved.  Exit status 0 = clean.
+#include <cstdio>
+#include <cstring>
+
+#include "flashbias.h"
+
+static fb_params good(int pass) {
+    static char buf[64]; // (never dereferenced by the checks)
+    fb_params p;
+    std::memset(&p, 0, sizeof(p));
+    p.size = sizeof(p);
+    p.dtype = FB_BF16;
+    p.B = 2; p.H = 4; p.Lq = 128; p.Lk = 96; p.d = 32; p.r = 8;
+    p.scale = 0.25f;
+    auto t = [&](int c) { return fb_tensor{buf, (int64_t)128 * 4 * c, c, 4 * c}; };
+    p.q = t(32); p.k = t(32); p.v = t(32); p.o = t(32);
+    p.q_bias = t(8); p.k_bias = t(8);
+    p.lse = reinterpret_cast<float *>(buf);
+    if (pass) {
+        p.dout = t(32); p.dq = t(32); p.dk = t(32); p.dv = t(32);
+        p.dq_bias = t(8); p.dk_bias = t(8);
+        p.delta = reinterpret_cast<float *>(buf);
+    }
+    return p;
+}
+
+int main() {
+    int bad = 0;
+    auto expect = [&](int got, int want, const char *what) {
+        if (got != want) {
+            std::fprintf(stderr, "%s: got %d, want %d (%s)\n", what, got, want, fb_last_error());
+            bad = 1;
+        }
+    };
+    for (int pass = 0; pass < 2; ++pass) {
+        fb_params p = good(pass);
+        expect(fb_check(&p, pass), FB_OK, "well-formed block");
+        p = good(pass); p.size = 8;                     expect(fb_check(&p, pass), FB_ERR_ABI, "size");
+        p = good(pass); p.dtype = FB_F32;               expect(fb_check(&p, pass), FB_ERR_DTYPE, "dtype");
+        p = good(pass); p.d = 129;                      expect(fb_check(&p, pass), FB_ERR_SHAPE, "d");
+        p = good(pass); p.Lk = -5;                      expect(fb_check(&p, pass), FB_ERR_SHAPE, "Lk");
+        p = good(pass); p.B = 1 << 20; p.H = 1 << 12;   expect(fb_check(&p, pass), FB_ERR_SHAPE, "grid");
+        p = good(pass); p.scale = 0.f;                  expect(fb_check(&p, pass), FB_ERR_SCALE, "scale");
+        p = good(pass); p.q.ptr = nullptr;              expect(fb_check(&p, pass), FB_ERR_NULL, "q");
+        p = good(pass); p.v.stride_s = -1;              expect(fb_check(&p, pass), FB_ERR_STRIDE, "v stride");
+        p = good(pass); p.mask_type = 7;                expect(fb_check(&p, pass), FB_ERR_MASK, "mask type");
+    }
+    expect(fb_check(nullptr, 0), FB_ERR_NULL, "null block");
+    fb_params p = good(1);
+    if (fb_bwd_workspace_bytes(&p) != (size_t)2 * 2 * 4 * 128 * sizeof(float)) bad = 1;
+    p.B = 0;
+    if (fb_bwd_workspace_bytes(&p) != 0 || fb_bwd_workspace_bytes(nullptr) != 0) bad = 1;
+    if (!bad) std::puts("sanitize_check: clean");
+    return bad;
+}

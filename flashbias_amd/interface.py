@@ -43,6 +43,15 @@ def _last_dim_contiguous(x):
 _FOLD_MIN_PAIRS = 1 << 29
 
 
+_MAX_RANK = 128  # FB_MAX_RANK of include/flashbias.h
+
+
+def _fold_keeps_rank_in_range(rank):
+    """One more factor column, padded to the next multiple of 8, must still be a rank the library
+    takes (rank 128 stays with the kernels' own vector-mask path)."""
+    return rank is None or -(-(rank + 1) // 8) * 8 <= _MAX_RANK
+
+
 def _fold_vector_mask(q, q_bias, k_bias, mask):
     """An additive (B|1, H|1, 1, Lk) mask is itself a rank-1 bias, 1_i * mask_j: appended to the
     factors as one more column it rides through the kernels' rank steps (which pad the rank to
@@ -61,27 +70,16 @@ def _fold_vector_mask(q, q_bias, k_bias, mask):
     return q_new, k_new
 
 
-def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
-    """Argument checks of _flash_attn_forward (flash_bias_triton.py:1100-1143) and the
-    parameter block shared by forward and backward.  Returns (params, keepalive)."""
-    batch, seqlen_q, nheads, d = q.shape
-    _, seqlen_k, _, _ = k.shape
-    assert k.shape == (batch, seqlen_k, nheads, d)
-    assert v.shape == (batch, seqlen_k, nheads, d)
-    assert d <= 128, "FlashBias only supports head dimensions up to 128"
-    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
-    assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
-    assert q.is_cuda and k.is_cuda and v.is_cuda
-    p = _lib.new_params()
-    p.dtype = _dtype_code(q.dtype)
-    p.B, p.H, p.Lq, p.Lk, p.d = batch, nheads, seqlen_q, seqlen_k, d
-    p.causal = int(bool(causal))
-    p.scale = softmax_scale or 1.0 / math.sqrt(d)
-    p.q, p.k, p.v = _tensor(q), _tensor(k), _tensor(v)
-    keep = []
+def _prepare_factors(q, k, q_bias, k_bias, mask):
+    """What the kernels get in place of (q_bias, k_bias, mask): a large vector mask folded into the
+    factors, the rank zero-padded to a multiple of 8, the channel dimension contiguous.  Done once
+    per forward; the backward reuses the result."""
+    batch, seqlen_q, nheads, _ = q.shape
+    seqlen_k = k.shape[1]
     if (mask is not None and mask.dim() == 4 and mask.shape[2] == 1 and mask.shape[3] == seqlen_k
             and mask.dtype == q.dtype and mask.is_cuda
-            and batch * nheads * seqlen_q * seqlen_k >= _FOLD_MIN_PAIRS):
+            and batch * nheads * seqlen_q * seqlen_k >= _FOLD_MIN_PAIRS
+            and _fold_keeps_rank_in_range(None if q_bias is None else q_bias.shape[-1])):
         q_bias, k_bias = _fold_vector_mask(q, q_bias, k_bias, mask)
         mask = None
     if q_bias is not None:
@@ -100,9 +98,39 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
             # the logits at |term| = 7000.
             pad = (0, (16 if rank < 8 else -(-rank // 8) * 8) - rank)
             q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
-            rank = q_bias.shape[-1]
         # (padding a permuted view keeps its permuted layout)
         q_bias, k_bias = _last_dim_contiguous(q_bias), _last_dim_contiguous(k_bias)
+    if mask is not None:
+        assert mask.dtype in (q.dtype, torch.float)
+        assert mask.is_cuda
+        assert mask.dim() == 4
+        if mask.stride(-1) != 1:
+            mask = mask.contiguous()
+    return q_bias, k_bias, mask
+
+
+def _prepare(q, k, v, factors, causal, softmax_scale):
+    """Argument checks of _flash_attn_forward (flash_bias_triton.py:1100-1143) and the
+    parameter block shared by forward and backward; `factors` = _prepare_factors(...).
+    Returns (params, keepalive)."""
+    q_bias, k_bias, mask = factors
+    batch, seqlen_q, nheads, d = q.shape
+    _, seqlen_k, _, _ = k.shape
+    assert k.shape == (batch, seqlen_k, nheads, d)
+    assert v.shape == (batch, seqlen_k, nheads, d)
+    assert d <= 128, "FlashBias only supports head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda
+    p = _lib.new_params()
+    p.dtype = _dtype_code(q.dtype)
+    p.B, p.H, p.Lq, p.Lk, p.d = batch, nheads, seqlen_q, seqlen_k, d
+    p.causal = int(bool(causal))
+    p.scale = softmax_scale or 1.0 / math.sqrt(d)
+    p.q, p.k, p.v = _tensor(q), _tensor(k), _tensor(v)
+    keep = []
+    if q_bias is not None:
+        rank = q_bias.shape[-1]
         # stride-0 broadcast over batch / heads (:1135-1136)
         qbe = q_bias.expand(batch, seqlen_q, nheads, rank)
         kbe = k_bias.expand(batch, seqlen_k, nheads, rank)
@@ -110,11 +138,6 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
         p.q_bias, p.k_bias = _tensor(qbe), _tensor(kbe)
         keep += [qbe, kbe]
     if mask is not None:
-        assert mask.dtype in (q.dtype, torch.float)
-        assert mask.is_cuda
-        assert mask.dim() == 4
-        if mask.stride(-1) != 1:
-            mask = mask.contiguous()
         if mask.shape[2:] == (1, seqlen_k):
             p.mask_type = _lib.FB_MASK_VECTOR
         elif mask.shape[2:] == (seqlen_q, seqlen_k):
@@ -128,13 +151,22 @@ def _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
     return p, keep
 
 
+def _params(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
+    """Parameter block for direct calls of the C ABI (tests, harness): (params, keepalive)."""
+    factors = _prepare_factors(q, k, q_bias, k_bias, mask)
+    p, keep = _prepare(q, k, v, factors, causal, softmax_scale)
+    return p, keep + [t for t in factors if t is not None]
+
+
 def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
-def _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
+def _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, factors=None):
     lib = _lib.load()
-    p, keep = _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+    if factors is None:
+        factors = _prepare_factors(q, k, q_bias, k_bias, mask)
+    p, keep = _prepare(q, k, v, factors, causal, softmax_scale)
     o = torch.empty_like(q)
     lse = torch.empty((p.B, p.H, p.Lq), device=q.device, dtype=torch.float32)
     p.o, p.lse = _tensor(o), lse.data_ptr()
@@ -144,10 +176,12 @@ def _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
     return o, lse, p.scale
 
 
-def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale):
+def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale, factors=None):
     lib = _lib.load()
     do = _last_dim_contiguous(do)
-    p, keep = _prepare(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+    if factors is None:
+        factors = _prepare_factors(q, k, q_bias, k_bias, mask)
+    p, keep = _prepare(q, k, v, factors, causal, softmax_scale)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     p.o, p.lse, p.dout = _tensor(o), lse.data_ptr(), _tensor(do)
     p.dq, p.dk, p.dv = _tensor(dq), _tensor(dk), _tensor(dv)
@@ -194,7 +228,10 @@ class FlashBiasFunc(torch.autograd.Function):
             q, k, v, q_bias, k_bias = [_last_dim_contiguous(x) for x in (q, k, v, q_bias, k_bias)]
         else:
             q, k, v = [_last_dim_contiguous(x) for x in (q, k, v)]
-        o, lse, ctx.softmax_scale = _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+        # (what the kernels consume in place of q_bias, k_bias, mask: kept for the backward)
+        ctx.kernel_factors = _prepare_factors(q, k, q_bias, k_bias, mask)
+        o, lse, ctx.softmax_scale = _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale,
+                                                        ctx.kernel_factors)
         ctx.save_for_backward(q, k, v, o, q_bias, k_bias, lse, mask)
         ctx.causal = causal
         return o
@@ -204,7 +241,7 @@ class FlashBiasFunc(torch.autograd.Function):
         q, k, v, o, q_bias, k_bias, lse, mask = ctx.saved_tensors
         assert not ctx.needs_input_grad[5], "FlashBias does not support mask gradient yet"
         dq, dk, dv, dq_bias, dk_bias = _flash_bias_backward(
-            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale)
+            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale, ctx.kernel_factors)
         return dq, dk, dv, dq_bias, dk_bias, None, None, None
 
 

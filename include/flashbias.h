@@ -9,13 +9,18 @@
  *   - Nothing here allocates or frees device memory: every buffer, including scratch
  *     (lse, delta), is owned by the caller, as in the reference where
  *     torch allocates o/lse/tmp/delta/dq_accum (flash_bias_triton.py:1145-1148, :1212-1219).
- *   - Launches are asynchronous on the given hipStream_t (passed as void*); no global
- *     mutable state, no autotuning side effects.
+ *   - Launches are asynchronous on the given hipStream_t (passed as void*); no autotuning side
+ *     effects.  The only process-wide state are write-once caches (compute units per device,
+ *     per-kernel occupancy and LDS limit; atomics, safe under concurrent first calls) and the
+ *     scratch array of fb_bwd_static.
  *   - Return value: FB_OK (0) or a negative fb_status; fb_last_error() gives the text of the
  *     last failure on the calling thread.  No C++ exception crosses the boundary.
  *   - Tensors use the reference layout (batch, seq, heads, channels) with the channel
- *     dimension contiguous; batch / head / seq are addressed through element strides, the
- *     way the Triton launchers pass them (flash_bias_triton.py:1163-1177).
+ *     dimension contiguous (stride 1: the ABI has no channel stride, a caller with another one
+ *     must make the tensor contiguous first, as the reference does, :1357-1360); batch / head /
+ *     seq are addressed through element strides, the way the Triton launchers pass them
+ *     (flash_bias_triton.py:1163-1177).  Sequence strides of 2^24 elements or more are correct
+ *     but take slower instantiations (the fast loaders keep a tile row's offset in 32 bits).
  */
 #ifndef FLASHBIAS_H
 #define FLASHBIAS_H
@@ -37,14 +42,14 @@ extern "C" {
 typedef enum fb_status {
     FB_OK = 0,
     FB_ERR_NULL = -1,       /* required pointer missing */
-    FB_ERR_SHAPE = -2,      /* non-positive size, d > 128, r > 128 */
+    FB_ERR_SHAPE = -2,      /* non-positive size, d > 128, r > 128, B * H * ceil(L / 32) >= 2^31 */
     FB_ERR_DTYPE = -3,      /* only fp16 / bf16 inputs (flash_bias_triton.py:1108) */
     FB_ERR_STRIDE = -4,     /* stride would alias gradient rows / negative stride */
     FB_ERR_MASK = -5,       /* bad mask type / dtype */
     FB_ERR_RESERVED = -6,
     FB_ERR_ABI = -7,        /* fb_params.size does not match this library */
     FB_ERR_LAUNCH = -8,     /* HIP reported a launch error */
-    FB_ERR_SCALE = -9       /* softmax scale not finite / not positive */
+    FB_ERR_SCALE = -9       /* softmax scale not finite or zero (negative scales are accepted) */
 } fb_status;
 
 typedef enum fb_dtype { FB_F16 = 0, FB_BF16 = 1, FB_F32 = 2 /* mask only */ } fb_dtype;

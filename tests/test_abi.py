@@ -75,6 +75,8 @@ def test_check_accepts_good_params():
     (lambda p: setattr(p.k_bias, "ptr", None), -1),
     (lambda p: setattr(p, "lse", None), -1),
     (lambda p: setattr(p.v, "stride_s", -32), -4),
+    (lambda p: setattr(p.k, "stride_s", 16), -4),  # rows of an input would overlap
+    (lambda p: setattr(p, "B", 1 << 20) or setattr(p, "H", 1 << 10), -2),  # grid beyond 2^31 - 1 workgroups
     (lambda p: setattr(p.o, "stride_b", 0), -4),
     (lambda p: setattr(p.o, "stride_s", 16), -4),
     (lambda p: setattr(p, "mask_type", 3), -5),
@@ -132,3 +134,26 @@ def test_operator_rejects_cpu_and_fp32_inputs():
         flash_bias_func(q.float(), q.float(), q.float())
     with pytest.raises(AssertionError):
         flash_bias_func(q, q[:, :4], q)
+
+
+def test_vector_mask_fold_respects_the_rank_limit():
+    """Folding a key-padding mask into the factors adds a column before the rank is padded to a
+    multiple of 8: rank 127 becomes 128, rank 128 would become 136, beyond what the library takes,
+    and keeps the kernels' own mask path."""
+    from flashbias_amd.interface import _fold_keeps_rank_in_range
+    assert _fold_keeps_rank_in_range(None) and _fold_keeps_rank_in_range(8) and _fold_keeps_rank_in_range(120)
+    assert _fold_keeps_rank_in_range(121) and _fold_keeps_rank_in_range(127)
+    assert not _fold_keeps_rank_in_range(128)
+
+
+def test_argument_checks_are_clean_under_sanitizers():
+    """fb_checks.cpp (fb_check, the size queries) rebuilt with -fsanitize=address,undefined and driven
+    with well-formed and malformed parameter blocks (flashbias_amd/csrc/sanitize_check.cpp)."""
+    import os
+    import subprocess
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "flashbias_amd", "csrc")
+    subprocess.check_call(["make", "-C", csrc, "sanitize"], stdout=subprocess.DEVNULL)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0")
+    res = subprocess.run([os.path.join(csrc, "build", "sanitize_check")], capture_output=True, text=True, env=env)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert "clean" in res.stdout

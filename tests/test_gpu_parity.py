@@ -306,14 +306,14 @@ def test_backward_phases_through_the_c_abi(gpu_device):
     the preprocess leaves -rowsum(o * dO) and lse * log2(e) in the scratch buffer (the delta of
     flash_bias_triton.py:358-400 with the sign and the scaling that the main kernels consume)."""
     from flashbias_amd import _lib
-    from flashbias_amd.interface import _prepare, _stream, _tensor
+    from flashbias_amd.interface import _params, _stream, _tensor
     dev = gpu_device
     B, L, H, d, r = 2, 333, 3, 32, 8
     q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=11)]
     lib = _lib.load()
 
     def params():
-        p, keep = _prepare(q, k, v, qb, kb, None, True, None)
+        p, keep = _params(q, k, v, qb, kb, None, True, None)
         bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, L), device=dev, dtype=torch.float32),
                     dq=torch.empty_like(q), dk=torch.empty_like(k), dv=torch.empty_like(v),
                     dqb=torch.empty((B, L, H, r), device=dev, dtype=q.dtype),

@@ -269,3 +269,16 @@ def test_blocked_ragged(causal, mask_kind):
 def test_blocked_broadcast_factors_and_no_bias():
     _check_blocked(2, 50, 50, 3, 16, 4, True, None, 16, 16, seed=23, bq=True, bk=True)
     _check_blocked(1, 33, 65, 2, 24, 0, False, None, 64, 32, seed=25)
+
+
+def test_c_oracle_is_clean_under_sanitizers():
+    """oracle/blocked.c rebuilt with -fsanitize=address,undefined and run on ragged, rectangular,
+    causal, masked and broadcast shapes with exactly sized buffers (oracle/sanitize_check.c)."""
+    import os
+    import subprocess
+    odir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "oracle")
+    subprocess.check_call(["make", "-C", odir, "sanitize"], stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:verify_asan_link_order=0")
+    res = subprocess.run([os.path.join(odir, "_sanitize", "sanitize_check")], capture_output=True, text=True, env=env)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert "clean" in res.stdout

@@ -10,7 +10,7 @@ def test_static_scratch_backward_matches_fb_bwd(gpu_device):
     """Two calls in a row, the second on a smaller input: every gradient and nothing else differs
     from what fb_bwd writes with a caller-owned scratch buffer (bit-exact: same kernels)."""
     from flashbias_amd import _lib
-    from flashbias_amd.interface import _prepare, _stream, _tensor
+    from flashbias_amd.interface import _params, _stream, _tensor
     dev = gpu_device
     lib = _lib.load()
 
@@ -18,7 +18,7 @@ def test_static_scratch_backward_matches_fb_bwd(gpu_device):
         q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=seed)]
 
         def params(with_scratch):
-            p, keep = _prepare(q, k, v, qb, kb, None, causal, None)
+            p, keep = _params(q, k, v, qb, kb, None, causal, None)
             bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, L), device=dev, dtype=torch.float32),
                         dq=torch.full_like(q, float("nan")), dk=torch.full_like(k, float("nan")),
                         dv=torch.full_like(v, float("nan")),
