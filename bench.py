@@ -106,7 +106,7 @@ def _phase_timers(w, dev):
         full = [torch.empty((p.B, L, p.H, p.r), device=dev, dtype=q.dtype) for L in (p.Lq, p.Lk)]
         p.dq_bias, p.dk_bias = _tensor(full[0]), _tensor(full[1])
         keep += full
-    delta = torch.empty((2,) + tuple(lse.shape), device=lse.device, dtype=torch.float32)  # -delta, lse*log2(e)
+    delta = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=lse.device, dtype=torch.float32)  # backward scratch
     p.delta = delta.data_ptr()
     keep += [o, lse, grads, delta]
 

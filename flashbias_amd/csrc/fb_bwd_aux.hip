@@ -1,6 +1,7 @@
 // delta = rowsum(o * dout), the memory-bound first step of the backward pass.  The scratch
-// buffer receives what the two main kernels consume: -delta in its first B*H*Lq floats and
-// lse * log2(e) in the next B*H*Lq.
+// buffer receives what the two main kernels consume: -delta in its first B*H*Lq floats,
+// lse * log2(e) in the next B*H*Lq, and both again as one chunk of 16-bit parts per query
+// (stat_chunk, from stat_offset on) for the streamlined dk/dv kernel.
 // Replaces _bwd_preprocess_do_o_dot of the reference (flash_bias/flash_bias_triton.py:358-400).
 #include "fb_kernels.h"
 
@@ -34,8 +35,10 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a) {
                 acc = __builtin_fmaf(T::to_float((uint16_t)(x[e] >> 16)), T::to_float((uint16_t)(y[e] >> 16)), acc);
             }
         }
+        const float l2 = a.lse[rix] * kLog2e;
         a.delta[rix] = -acc;
-        a.delta[rows + rix] = a.lse[rix] * kLog2e;
+        a.delta[rows + rix] = l2;
+        reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[rix] = stat_chunk<T>(-acc, l2);
     }
 }
 
@@ -73,8 +76,10 @@ __global__ __launch_bounds__(256) void bwd_preprocess_chunks_kernel(const BwdArg
         for (int m = 1; m < CH; m <<= 1) acc += __shfl_xor(acc, m, 64);
         if (c == 0) {
             const int64_t rix = ((int64_t)b * a.H + h) * a.Lq + i;
+            const float l2 = a.lse[rix] * kLog2e;
             a.delta[rix] = -acc;
-            a.delta[rows + rix] = a.lse[rix] * kLog2e;
+            a.delta[rows + rix] = l2;
+            reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[rix] = stat_chunk<T>(-acc, l2);
         }
     }
 }

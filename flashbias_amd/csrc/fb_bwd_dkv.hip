@@ -230,8 +230,7 @@ struct DkvDirect {
 };
 
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
-bwd_dkv_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
 
@@ -555,6 +554,12 @@ bwd_dkv_kernel(const BwdArgs a) {
     }
 }
 
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
+bwd_dkv_kernel(const BwdArgs a) {
+    bwd_dkv_body<T, C>(a);
+}
+
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART, bool FOLD>
 static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
     typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK, PART, FOLD> C;
@@ -590,6 +595,10 @@ static hipError_t launch_dkv_vec(const BwdArgs &a, hipStream_t stream) {
     }
 }
 
+} // namespace fb
+#include "fb_bwd_dkv_lean.h"
+namespace fb {
+
 template <class T, int NKD, int NKR, int NDV>
 static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
     // the direct loader keeps the byte distance between two steps' rows in 32 bits
@@ -600,6 +609,11 @@ static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
     if (a.mask.type)
         return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_dkv_vec<T, NKD, NKR, NDV, false, true>(a, stream);
+    if constexpr (NKD == 2 && NKR <= 1 && NDV == 1) {
+        // the streamlined kernel, where its 128-key workgroups fill the chip's two slots per CU
+        const int64_t wgs = (int64_t)a.B * a.H * ((a.Lk + 127) / 128);
+        if (vec && dkv_lean_ok(a) && wgs >= 2 * num_cus()) return launch_dkv_lean<T, NKR>(a, stream);
+    }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lq)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
     }

@@ -164,9 +164,9 @@ struct DqDirect {
     int m0_ = 0; // first query of the workgroup (set by init_mask)
 };
 
+// The whole dq / dq_bias computation of one workgroup; the kernel below is nothing else.
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::QBLK == 1 && C::NK <= 3 ? 1 : 0)))) void
-bwd_dq_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
 
@@ -253,8 +253,10 @@ bwd_dq_kernel(const BwdArgs a) {
             nd = ok ? -part : 0.f;
             l2 = ok ? a.lse[sidx] * kLog2e : INFINITY;
             if (ok && g == 0) {
+                const int64_t rows = (int64_t)a.B * a.H * a.Lq;
                 a.delta[sidx] = nd;
-                a.delta[(int64_t)a.B * a.H * a.Lq + sidx] = l2;
+                a.delta[rows + sidx] = l2;
+                reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[sidx] = stat_chunk<T>(nd, l2);
             }
         } else {
             // the preprocess step left -delta and lse * log2(e) in the scratch buffer
@@ -478,6 +480,12 @@ bwd_dq_kernel(const BwdArgs a) {
                 }
         }
     }
+}
+
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::QBLK == 1 && C::NK <= 3 ? 1 : 0)))) void
+bwd_dq_kernel(const BwdArgs a) {
+    bwd_dq_body<T, C>(a);
 }
 
 template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2, bool FOLD, bool KB1 = false>

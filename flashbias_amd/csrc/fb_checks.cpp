@@ -61,7 +61,7 @@ const char *fb_last_error(void) { return g_err; }
 
 size_t fb_bwd_workspace_bytes(const fb_params *p) {
     if (!p || p->B <= 0 || p->H <= 0 || p->Lq <= 0) return 0;
-    return (size_t)2 * (size_t)p->B * (size_t)p->H * (size_t)p->Lq * sizeof(float);
+    return fb::bwd_scratch_bytes((int64_t)p->B * p->H * p->Lq);
 }
 
 int fb_check(const fb_params *p, int pass) {
@@ -107,6 +107,7 @@ int fb_check(const fb_params *p, int pass) {
         if ((rc = check_out(p->dk_bias, p->r, p->B, p->H, p->Lk, "dk_bias"))) return rc;
     }
     if (!p->delta) return fail(FB_ERR_NULL, "%s: null pointer", "delta");
+    if (reinterpret_cast<uintptr_t>(p->delta) % 16 != 0) return fail(FB_ERR_STRIDE, "%s: must be 16-byte aligned", "delta");
     return FB_OK;
 }
 

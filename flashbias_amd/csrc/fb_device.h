@@ -150,6 +150,43 @@ __device__ __forceinline__ u32x4_t fold_scale_chunk(u32x4_t x, float inv, bool s
     return out;
 }
 
+// True if any of the eight 16-bit values of a chunk is +-inf (or NaN).
+template <class T>
+__device__ __forceinline__ bool chunk_has_inf(u32x4_t x) {
+    bool bad = false;
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const float f = T::to_float((uint16_t)(hf ? x[e] >> 16 : x[e] & 0xffffu));
+            bad |= !(fabsf(f) <= 3.0e38f);
+        }
+    return bad;
+}
+
+// Per-query statistics of the backward pass as one 16-byte chunk of eight 16-bit values:
+// -lse * log2(e) in k-slots 0..2 and -delta in k-slots 3..5, each as three parts (the value
+// rounded to 16 bits, then twice the rounded remainder: 24 significant bits for bf16), zeros in
+// slots 6, 7.  An MFMA step against ones in slots 0..2 (or 3..5) adds the value to an accumulator,
+// which is how the streamlined backward kernels subtract lse and delta without touching the VALU.
+// nd = -delta, l2 = lse * log2(e).
+template <class T>
+__device__ __forceinline__ u32x4_t stat_chunk(float nd, float l2) {
+    uint32_t p[6];
+    // (the values as they are stored in fp32, not an expression the compiler may still fuse into the
+    // subtractions below: every writer of the scratch buffer must produce the same bits)
+    asm volatile("" : "+v"(nd), "+v"(l2));
+    float x = -l2;
+#pragma unroll
+    for (int i = 0; i < 6; ++i) {
+        if (i == 3) x = nd;
+        const uint16_t hi = T::from_float(x);
+        p[i] = hi;
+        x -= T::to_float(hi);
+    }
+    return u32x4_t{p[0] | (p[1] << 16), p[2] | (p[3] << 16), p[4] | (p[5] << 16), 0u};
+}
+
 // Position of key (or query) `x` of a 16-group inside an LDS row that feeds the A operand
 // of an MFMA whose B operand comes straight from a C-layout register block: C rows
 // 8b + 4g + c (b, g in {0,1}) must sit at slot 8g + 4b + c, i.e. bits 2 and 3 swap.

@@ -584,7 +584,7 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
     if constexpr (NKD == 2 && NKR <= 1 && NDV == 1) {
         // the streamlined kernel has 256-query workgroups only: grids that fill the chip (see launch_fwd_vec)
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (vec && fwd_lean_ok(a) && wgs >= (int64_t)(a.causal ? 7 : 2) * num_cus())
+        if (vec && fwd_lean_ok(a) && wgs >= (int64_t)2 * num_cus())
             return launch_fwd_lean<T, NKR>(a, stream);
     }
     if constexpr (NKR <= 2) {

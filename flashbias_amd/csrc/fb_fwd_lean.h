@@ -1,5 +1,5 @@
 // Streamlined forward kernel for the shapes the benchmark family lives on: aligned tensors, no
-// additive mask, head dim <= 32, rank <= 8 (or no factors), grids that fill the chip.  Included by
+// additive or causal mask, head dim 32, rank 8 (or no factors), grids that fill the chip.  Included by
 // fb_fwd.hip after the general kernel.  What differs from fwd_kernel is the arithmetic per score
 // and the way tiles reach LDS:
 //
@@ -26,6 +26,8 @@
 // Per score the VALU is left with exp2, the row-sum add and half a convert.
 #pragma once
 #include <type_traits>
+
+#include "fb_lean_tiles.h"
 
 namespace fb {
 
@@ -62,12 +64,6 @@ __device__ __attribute__((noinline)) void fwd_lean_retry() {
     fwd_body<T, typename C::General>(a);
 }
 
-// 16 bytes per lane from base + off (base wave-uniform, off a 32-bit byte offset per lane) to LDS
-// byte address lds + 16 * lane; every lane of the wave takes part.
-__device__ __forceinline__ void lds_dma16_all(uint32_t off, const void *base, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"(lds) : "memory");
-}
-
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void fwd_lean_kernel(const FwdArgs a) {
     constexpr int NK = C::NK, NKD = C::NKD, NKR = C::NKR;
@@ -80,8 +76,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int total = a.ntiles_m * a.B * a.H;
     const int work = xcd_remap(blockIdx.x, total);
     const int bh = work / a.ntiles_m;
-    int tile_m = work % a.ntiles_m;
-    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
+    const int tile_m = work % a.ntiles_m;
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
     const int wq0 = m0 + wave * 64; // first query of this wave
@@ -109,9 +104,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
             qbr[qb][0] = fold_scale_chunk<T>(load_chunk<true>(qbbase, a.qb.ss, query, a.Lq, 0, a.r), kLog2e, true, g == 1);
     }
 
-    int k_end = a.Lk;
-    if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
-    const int ntiles_k = (k_end + C::BN - 1) / C::BN;
+    const int ntiles_k = (a.Lk + C::BN - 1) / C::BN;
 
     // ---- the copies.  This lane's place in an instruction's 8 lines and what belongs there
     const int dline = lane >> 3, dslot = (lane & 7) ^ ((lane >> 4) & 3);
@@ -194,13 +187,12 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         if constexpr (NKR > 0) acc = T::mfma(f[NKD], qbr[qb][0], acc);
         return acc;
     };
-    // -inf for keys past the end and pairs that a causal mask hides
-    auto hide = [&](f32x16_t &s, int ns, int qb) {
-        const int query = wq0 + 32 * qb + c;
+    // -inf for keys past the end
+    auto hide = [&](f32x16_t &s, int ns) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = ns + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (key >= a.Lk || (a.causal && key > query)) s[v] = -INFINITY;
+            if (key >= a.Lk) s[v] = -INFINITY;
         }
     };
 
@@ -251,7 +243,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             f32x16_t s = scores(ka, qb, zero16);
-            hide(s, 0, qb);
+            hide(s, 0);
 #pragma unroll
             for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[v]);
             l_run[qb] = 0.f;
@@ -271,7 +263,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         const int n0 = it * C::BN;
         take_turn(turn, a.slots);
         if (it + 2 < ntiles_k) issue((STG + 2) % 3, n0 + 2 * C::BN);
-        const bool edge = n0 + C::BN > a.Lk || (a.causal && n0 + C::BN - 1 > wq0);
+        const bool edge = n0 + C::BN > a.Lk;
         f32x16_t s_cur, s_nxt;
         read_ka(ka, STG, 0);
         s_cur = scores(ka, 0, minit);
@@ -281,12 +273,12 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
             if (kb + 1 < C::KB) read_ka(nxt, STG, kb + 1);
             read_va(va, STG, kb);
             s_nxt = scores(cur, 1, minit);
-            if (hidden_pairs) hide(s_cur, n0 + 32 * kb, 0);
+            if (hidden_pairs) hide(s_cur, n0 + 32 * kb);
             softmax_pv(s_cur, va, 0);
             s_cur = s_nxt;
             interleave();
             if (kb + 1 < C::KB) s_nxt = scores(nxt, 0, minit);
-            if (hidden_pairs) hide(s_cur, n0 + 32 * kb, 1);
+            if (hidden_pairs) hide(s_cur, n0 + 32 * kb);
             softmax_pv(s_cur, va, 1);
             s_cur = s_nxt;
             interleave();
@@ -297,7 +289,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                 key_block(ka, kn, kb, false);
                 key_block(kn, ka, kb + 1, false);
             }
-        } else { // the same with the hidden pairs of every block set to -inf (p = 0)
+        } else { // the ragged last tile: the same with the keys past the end set to -inf (p = 0)
 #pragma unroll
             for (int kb = 0; kb < C::KB; kb += 2) {
                 key_block(ka, kn, kb, true);
@@ -358,10 +350,15 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 // no zero padding of the channels); the factors then fit the hi + lo layout of one bias step.  The bounds
 // on the scale keep the folded operands away from the ends of fp32's range; what a 16-bit type
 // cannot hold after the scaling ends up as inf / NaN row sums, which take the fallback.
+// Not for causal calls nor for fewer than 128 keys: with a reference point that is not the row's
+// own maximum the largest P of a row is not exactly 1, so a row that sees one or two keys comes
+// out an ulp off v (the general kernel returns it exactly), and the reference point of a query
+// depends on keys that only the other query of its lane may see, which breaks the bit-for-bit
+// independence of o[i] from keys j > i.
 inline bool fwd_lean_ok(const FwdArgs &a) {
     const int64_t lim = (int64_t)1 << 24; // (32-bit tile row offsets in the copies)
-    return a.d == 32 && (a.r == 8 || a.r == 0) && a.scale > 1e-6f && a.scale < 1e6f && a.k.ss < lim && a.v.ss < lim &&
-           (a.r == 0 || a.kb.ss < lim);
+    return a.d == 32 && (a.r == 8 || a.r == 0) && !a.causal && a.Lk >= 128 && a.scale > 1e-6f && a.scale < 1e6f &&
+           a.k.ss < lim && a.v.ss < lim && (a.r == 0 || a.kb.ss < lim);
 }
 
 template <class T, int NKR>

@@ -1,6 +1,8 @@
 // Host-visible kernel argument blocks and launchers (implemented in fb_fwd.hip / fb_bwd.hip).
 #pragma once
 #include <atomic>
+
+#include "fb_checks.h"
 #include <cmath>
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -25,7 +27,7 @@ struct BwdArgs {
     Tensor dq, dk, dv, dqb, dkb;
     MaskDesc mask;
     const float *lse; // (B, H, Lq)
-    float *delta;     // (B, H, Lq)
+    float *delta;     // scratch: -delta (B, H, Lq), lse * log2(e) (B, H, Lq), then one stat_chunk per query at stat_offset()
     int B, H, Lq, Lk, d, r;
     int causal;
     float scale;

@@ -7,7 +7,7 @@
 #include "flashbias.h"
 
 static fb_params good(int pass) {
-    static char buf[64]; // (never dereferenced by the checks)
+    alignas(16) static char buf[64]; // (never dereferenced by the checks)
     fb_params p;
     std::memset(&p, 0, sizeof(p));
     p.size = sizeof(p);
@@ -46,10 +46,14 @@ int main() {
         p = good(pass); p.q.ptr = nullptr;              expect(fb_check(&p, pass), FB_ERR_NULL, "q");
         p = good(pass); p.v.stride_s = -1;              expect(fb_check(&p, pass), FB_ERR_STRIDE, "v stride");
         p = good(pass); p.mask_type = 7;                expect(fb_check(&p, pass), FB_ERR_MASK, "mask type");
+        if (pass) {
+            p = good(pass); p.delta = reinterpret_cast<float *>(reinterpret_cast<char *>(p.delta) + 4);
+            expect(fb_check(&p, pass), FB_ERR_STRIDE, "scratch alignment");
+        }
     }
     expect(fb_check(nullptr, 0), FB_ERR_NULL, "null block");
     fb_params p = good(1);
-    if (fb_bwd_workspace_bytes(&p) != (size_t)2 * 2 * 4 * 128 * sizeof(float)) bad = 1;
+    if (fb_bwd_workspace_bytes(&p) != (size_t)2 * 4 * 128 * (2 * sizeof(float) + 16)) bad = 1; // per query row: two floats, one chunk
     p.B = 0;
     if (fb_bwd_workspace_bytes(&p) != 0 || fb_bwd_workspace_bytes(nullptr) != 0) bad = 1;
     if (!bad) std::puts("sanitize_check: clean");

@@ -36,7 +36,7 @@ extern "C" {
 #define FB_MAX_HEADDIM 128 /* flash_bias_triton.py:1106 */
 #define FB_MAX_RANK 128
 /* Size of the library-owned scratch buffer used by fb_bwd_static (one copy per GPU, held until the
- * process ends): enough for B * H * Lq <= 4194304 query rows. */
+ * process ends): enough for B * H * Lq <= 1398101 query rows (24 bytes each). */
 #define FB_STATIC_SCRATCH_BYTES (32u << 20)
 
 typedef enum fb_status {
@@ -86,7 +86,8 @@ typedef struct fb_params {
     fb_tensor dq, dk, dv;       /* bwd out */
     fb_tensor dq_bias, dk_bias; /* bwd out, full (B, L, H, r) shape: the caller reduces over
                                    broadcast dims */
-    float *delta;               /* (2, B, H, Lq) fp32 scratch, written by the backward: -delta, lse * log2(e) */
+    float *delta;               /* backward scratch of fb_bwd_workspace_bytes() bytes, 16-byte aligned, written by the
+                                   backward: -delta and lse * log2(e) per query row, as fp32 and as 16-bit parts */
 } fb_params;
 
 /* Library / ABI version. */
@@ -100,7 +101,8 @@ const char *fb_last_error(void);
  * pass: 0 = forward, 1 = backward. */
 int fb_check(const fb_params *p, int pass);
 
-/* Bytes of the backward's scratch buffer fb_params.delta for these sizes (2 * B * H * Lq floats;
+/* Bytes of the backward's scratch buffer fb_params.delta for these sizes (24 per query row: two
+ * floats and one 16-byte chunk of 16-bit parts, the second array starting on a 16-byte boundary;
  * the reference allocates delta, dq_accum and dq_bias_accum itself, flash_bias_triton.py:1212-1219).
  * Only B, H and Lq are read; returns 0 for a null pointer or non-positive sizes. */
 size_t fb_bwd_workspace_bytes(const fb_params *p);
@@ -133,7 +135,9 @@ int fb_bwd_static(const fb_params *p, void *stream);
 /* The backward in three phases, exported so that a harness can time them separately (call them in
  * this order: the two main kernels read what the preprocess wrote).
  *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400); fills the
- *                      scratch with -delta (first B*H*Lq floats) and lse * log2(e) (next B*H*Lq)
+ *                      scratch with -delta (first B*H*Lq floats), lse * log2(e) (next B*H*Lq) and, from the
+ *                      next 16-byte boundary on, both once more per query row as three 16-bit parts each
+ *                      (what the streamlined dk/dv kernel feeds to its MFMAs)
  *   fb_bwd_dkv:        recompute P from lse; dk, dv, dk_bias, one workgroup per key tile
  *                      (_bwd_kernel / _bwd_kernel_one_col_block, :450-1097, minus dq)
  *   fb_bwd_dq:         recompute P from lse; dq, dq_bias, one workgroup per query tile

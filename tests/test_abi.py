@@ -32,7 +32,10 @@ def test_workspace_size_query():
     lib = _lib.load()
     p = _lib.new_params()
     p.B, p.H, p.Lq = 2, 4, 1000
-    assert lib.fb_bwd_workspace_bytes(p) == 2 * 2 * 4 * 1000 * 4
+    # per query row: -delta and lse * log2(e) as floats, then one 16-byte chunk of 16-bit parts
+    assert lib.fb_bwd_workspace_bytes(p) == 2 * 4 * 1000 * (2 * 4 + 16)
+    p.Lq = 1001  # the chunks start 16-byte aligned
+    assert lib.fb_bwd_workspace_bytes(p) == (2 * 8008 + 3) // 4 * 4 * 4 + 8008 * 16
     p.Lq = 0
     assert lib.fb_bwd_workspace_bytes(p) == 0
     assert lib.fb_bwd_workspace_bytes(None) == 0

@@ -318,7 +318,8 @@ def test_backward_phases_through_the_c_abi(gpu_device):
                     dq=torch.empty_like(q), dk=torch.empty_like(k), dv=torch.empty_like(v),
                     dqb=torch.empty((B, L, H, r), device=dev, dtype=q.dtype),
                     dkb=torch.empty((B, L, H, r), device=dev, dtype=q.dtype),
-                    scratch=torch.full((2, B, H, L), float("nan"), device=dev, dtype=torch.float32))
+                    scratch=torch.full((lib.fb_bwd_workspace_bytes(p) // 4,), float("nan"), device=dev,
+                                       dtype=torch.float32))
         p.o, p.lse, p.dout = _tensor(bufs["o"]), bufs["lse"].data_ptr(), _tensor(do)
         p.dq, p.dk, p.dv = _tensor(bufs["dq"]), _tensor(bufs["dk"]), _tensor(bufs["dv"])
         p.dq_bias, p.dk_bias, p.delta = _tensor(bufs["dqb"]), _tensor(bufs["dkb"]), bufs["scratch"].data_ptr()
@@ -336,8 +337,17 @@ def test_backward_phases_through_the_c_abi(gpu_device):
         assert torch.equal(whole[name], parts[name]), name
     o, lse = whole["o"].float(), whole["lse"]
     delta = (o * do.float()).sum(-1).permute(0, 2, 1)  # (B, H, L)
-    assert torch.allclose(whole["scratch"][0], -delta, rtol=1e-5, atol=1e-5)
-    assert torch.allclose(whole["scratch"][1], lse * math.log2(math.e), rtol=1e-6, atol=1e-6)
+    n = B * H * L
+    stats = whole["scratch"][:2 * n].view(2, B, H, L)
+    assert torch.allclose(stats[0], -delta, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(stats[1], lse * math.log2(math.e), rtol=1e-6, atol=1e-6)
+    # the same two values once more per query, as three 16-bit parts each (what the streamlined dk/dv
+    # kernel feeds to its MFMAs): -lse * log2(e) in elements 0..2, -delta in 3..5, zeros in 6, 7
+    off = (2 * n + 3) // 4 * 4
+    parts = whole["scratch"][off:off + 4 * n].view(torch.bfloat16).view(B, H, L, 8).float()
+    assert torch.allclose(parts[..., 0:3].sum(-1), -stats[1], rtol=1e-6, atol=1e-6)
+    assert torch.allclose(parts[..., 3:6].sum(-1), stats[0], rtol=1e-6, atol=1e-6)
+    assert (parts[..., 6:] == 0).all()
 
 
 @pytest.mark.parametrize("Lq,Lk", [(1000, 1000), (777, 1300), (1300, 777)])
@@ -356,6 +366,19 @@ def test_large_grids_ragged(gpu_device, B, H, Lq, Lk, r, causal):
     cases above never reach; ragged last tiles, rectangular and causal shapes."""
     assert B * H * ((Lq + 255) // 256) >= (3 if causal else 2) * 256
     _case(gpu_device, B, Lq, Lk, H, 32, r, torch.bfloat16, causal, seed=13)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("r", [0, 8])
+@pytest.mark.parametrize("causal", [False, True])
+def test_streamlined_kernels(gpu_device, dtype, r, causal):
+    """Head dim 32, rank 8 or no factors, aligned, unmasked, on grids that fill an MI355X: the shapes
+    that take the streamlined forward kernel (not causal, at least two 256-query workgroups per
+    compute unit) and the streamlined dk/dv kernel (at least two 128-key workgroups per compute
+    unit), with ragged last tiles on both sides, in both element types."""
+    B, H, Lq, Lk = (8, 32, 1800, 600) if causal else (8, 16, 1000, 1000)
+    assert B * H * ((Lq + 255) // 256) >= 2 * 256 and B * H * ((Lk + 127) // 128) >= 2 * 256
+    _case(gpu_device, B, Lq, Lk, H, 32, r, dtype, causal, seed=14)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
