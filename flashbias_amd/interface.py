@@ -158,11 +158,29 @@ def _params(q, k, v, q_bias, k_bias, mask, causal, softmax_scale):
     return p, keep + [t for t in factors if t is not None]
 
 
-def _stream():
-    return torch.cuda.current_stream().cuda_stream
+def _stream(device=None):
+    """Raw handle of torch's current stream on `device` (default: the current device)."""
+    index = torch.cuda.current_device() if device is None or device.index is None else device.index
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+def _launch(fn, p, device):
+    """One C-ABI call on torch's current stream of `device`, with that device current."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        _lib.check_status(fn(p, _stream(device)))
+    else:
+        with torch.cuda.device(device):
+            _lib.check_status(fn(p, _stream(device)))
 
 
 def _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, factors=None):
+    """(o, lse, softmax_scale), as _flash_attn_forward of the reference (flash_bias_triton.py:1100-1194)."""
+    return _forward_with_block(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, factors)[:3]
+
+
+def _forward_with_block(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, factors=None):
+    """Returns (o, lse, softmax_scale, block): block = the parameter block of the call and the
+    tensors its pointers refer to, which a backward over the same tensors may reuse."""
     lib = _lib.load()
     if factors is None:
         factors = _prepare_factors(q, k, q_bias, k_bias, mask)
@@ -170,18 +188,19 @@ def _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, fa
     o = torch.empty_like(q)
     lse = torch.empty((p.B, p.H, p.Lq), device=q.device, dtype=torch.float32)
     p.o, p.lse = _tensor(o), lse.data_ptr()
-    with torch.cuda.device(q.device):
-        _lib.check_status(lib.fb_fwd(p, _stream()))
-    del keep
-    return o, lse, p.scale
+    _launch(lib.fb_fwd, p, q.device)
+    return o, lse, p.scale, (p, keep)
 
 
-def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale, factors=None):
+def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale, factors=None, block=None):
     lib = _lib.load()
     do = _last_dim_contiguous(do)
-    if factors is None:
-        factors = _prepare_factors(q, k, q_bias, k_bias, mask)
-    p, keep = _prepare(q, k, v, factors, causal, softmax_scale)
+    if block is not None and (block[0].q.ptr, block[0].k.ptr, block[0].v.ptr) == (q.data_ptr(), k.data_ptr(), v.data_ptr()):
+        p, keep = block  # the forward's block: same tensors (the factors and the mask are kept alive by it)
+    else:
+        if factors is None:
+            factors = _prepare_factors(q, k, q_bias, k_bias, mask)
+        p, keep = _prepare(q, k, v, factors, causal, softmax_scale)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     p.o, p.lse, p.dout = _tensor(o), lse.data_ptr(), _tensor(do)
     p.dq, p.dk, p.dv = _tensor(dq), _tensor(dk), _tensor(dv)
@@ -193,8 +212,7 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     # scratch of the backward: -delta and lse * log2(e), sized by the library
     delta = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=lse.device, dtype=torch.float32)
     p.delta = delta.data_ptr()
-    with torch.cuda.device(q.device):
-        _lib.check_status(lib.fb_bwd(p, _stream()))
+    _launch(lib.fb_bwd, p, q.device)
     del keep
     dq_bias = dk_bias = None
     if q_bias is not None:
@@ -230,8 +248,8 @@ class FlashBiasFunc(torch.autograd.Function):
             q, k, v = [_last_dim_contiguous(x) for x in (q, k, v)]
         # (what the kernels consume in place of q_bias, k_bias, mask: kept for the backward)
         ctx.kernel_factors = _prepare_factors(q, k, q_bias, k_bias, mask)
-        o, lse, ctx.softmax_scale = _flash_bias_forward(q, k, v, q_bias, k_bias, mask, causal, softmax_scale,
-                                                        ctx.kernel_factors)
+        o, lse, ctx.softmax_scale, ctx.block = _forward_with_block(q, k, v, q_bias, k_bias, mask, causal,
+                                                                   softmax_scale, ctx.kernel_factors)
         ctx.save_for_backward(q, k, v, o, q_bias, k_bias, lse, mask)
         ctx.causal = causal
         return o
@@ -241,7 +259,7 @@ class FlashBiasFunc(torch.autograd.Function):
         q, k, v, o, q_bias, k_bias, lse, mask = ctx.saved_tensors
         assert not ctx.needs_input_grad[5], "FlashBias does not support mask gradient yet"
         dq, dk, dv, dq_bias, dk_bias = _flash_bias_backward(
-            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale, ctx.kernel_factors)
+            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale, ctx.kernel_factors, ctx.block)
         return dq, dk, dv, dq_bias, dk_bias, None, None, None
 
 
