@@ -610,9 +610,10 @@ static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
         return vec ? launch_dkv_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_dkv_vec<T, NKD, NKR, NDV, false, true>(a, stream);
     if constexpr (NKD == 2 && NKR <= 1 && NDV == 1) {
-        // the streamlined kernel, where its 128-key workgroups fill the chip's two slots per CU
-        const int64_t wgs = (int64_t)a.B * a.H * ((a.Lk + 127) / 128);
-        if (vec && dkv_lean_ok(a) && wgs >= 2 * num_cus()) return launch_dkv_lean<T, NKR>(a, stream);
+        // the streamlined kernel: same 128-key workgroups as the general one, and ahead of it at every
+        // grid size (measured at B2 H4: 0.019 against 0.023 ms at L=1024, 0.063 against 0.082 at 4096,
+        // 0.73 against 0.82 at 16384)
+        if (vec && dkv_lean_ok(a)) return launch_dkv_lean<T, NKR>(a, stream);
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lq)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
