@@ -13,7 +13,7 @@ FB_F16, FB_BF16, FB_F32 = 0, 1, 2
 FB_MASK_NONE, FB_MASK_VECTOR, FB_MASK_MATRIX = 0, 1, 2
 
 #: every symbol that include/flashbias.h declares
-EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_check", "fb_fwd", "fb_bwd",
+EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_check", "fb_fwd", "fb_bwd", "fb_sum_over_batch",
            "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static")
 
 
@@ -67,6 +67,9 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = [ctypes.POINTER(FbParams), ctypes.c_void_p]
         fn.restype = ctypes.c_int
+    lib.fb_sum_over_batch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
+                                      ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]
+    lib.fb_sum_over_batch.restype = ctypes.c_int
     _lib = lib
     return lib
 

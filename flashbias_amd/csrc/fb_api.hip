@@ -190,6 +190,20 @@ int fb_bwd_dq(const fb_params *p, void *stream) {
                     "fb_bwd_dq");
 }
 
+int fb_sum_over_batch(const void *full, void *out, int dtype, int out_dtype, int64_t B, int64_t n, int64_t batch_stride,
+                      void *stream) {
+    fb::api_clear_error();
+    if (!full || !out) return fb::api_fail(FB_ERR_NULL, "fb_sum_over_batch: null pointer");
+    if (dtype != FB_F16 && dtype != FB_BF16) return fb::api_fail(FB_ERR_DTYPE, "only fp16 and bf16 are supported");
+    if (out_dtype != dtype && out_dtype != FB_F32) return fb::api_fail(FB_ERR_DTYPE, "output must have the input dtype or fp32");
+    if (B <= 0 || n <= 0 || (n + 63) / 64 > 0x7fffffff) return fb::api_fail(FB_ERR_SHAPE, "B and n must be positive (n below 2^37)");
+    if (n % 8 != 0 || batch_stride % 8 != 0 || batch_stride < n || reinterpret_cast<uintptr_t>(full) % 16 != 0)
+        return fb::api_fail(FB_ERR_STRIDE, "fb_sum_over_batch: rows must be 16-byte aligned multiples of 8 elements that do not overlap");
+    return launched(fb::launch_sum_over_batch(full, out, dtype == FB_BF16, out_dtype == FB_F32, B, n, batch_stride,
+                                              static_cast<hipStream_t>(stream)),
+                    "fb_sum_over_batch");
+}
+
 int fb_bwd_static(const fb_params *p, void *stream) {
     // fb_bwd with the scratch buffer taken from the library's own static device array instead of
     // fb_params.delta (which is ignored): no allocation, here or in anything it calls.

@@ -3,6 +3,8 @@
 // lse * log2(e) in the next B*H*Lq, and both again as one chunk of 16-bit parts per query
 // (stat_chunk, from stat_offset on) for the streamlined dk/dv kernel.
 // Replaces _bwd_preprocess_do_o_dot of the reference (flash_bias/flash_bias_triton.py:358-400).
+// Also here: the sum over the batch of a full-shape factor gradient, the memory-bound last step
+// of the backward pass for factors that all batch entries share.
 #include "fb_kernels.h"
 
 namespace fb {
@@ -116,6 +118,60 @@ static void launch_preprocess_t(const BwdArgs &a, hipStream_t stream) {
     if (blocks > 65536) blocks = 65536;
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(bwd_preprocess_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+}
+
+// out[j] = sum over b of full[b * sb + j], j < n (a multiple of 8), fp32 accumulation in a fixed
+// order: every thread adds the rows b = lane, lane + 32, ... of its 8 columns, then the 32 partial
+// sums of a column are added in lane order.  One workgroup owns 64 consecutive columns (128 bytes
+// of every row: whole cache lines) and streams down all rows, 32 rows per pass.
+template <class T, bool OUT_F32>
+__global__ __launch_bounds__(256) void sum_over_batch_kernel(const uint16_t *full, void *out, int64_t B, int64_t n, int64_t sb) {
+    __shared__ float part[32][65]; // (65: the column sums below walk down a column of this array)
+    const int cg = threadIdx.x & 7, rl = threadIdx.x >> 3;
+    const int64_t col = (int64_t)blockIdx.x * 64 + cg * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (col < n) {
+        const uint16_t *p = full + col;
+#pragma unroll 4
+        for (int64_t b = rl; b < B; b += 32) {
+            const u32x4_t x = *reinterpret_cast<const u32x4_t *>(p + b * sb);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                acc[2 * e] += T::to_float((uint16_t)(x[e] & 0xffffu));
+                acc[2 * e + 1] += T::to_float((uint16_t)(x[e] >> 16));
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[rl][cg * 8 + e] = acc[e];
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        const int64_t j = (int64_t)blockIdx.x * 64 + threadIdx.x;
+        float s = 0.f;
+#pragma unroll
+        for (int r = 0; r < 32; ++r) s += part[r][threadIdx.x];
+        if (j < n) {
+            if (OUT_F32)
+                static_cast<float *>(out)[j] = s;
+            else
+                static_cast<uint16_t *>(out)[j] = T::from_float(s);
+        }
+    }
+}
+
+hipError_t launch_sum_over_batch(const void *full, void *out, bool bf16, bool out_f32, int64_t B, int64_t n, int64_t sb,
+                                 hipStream_t stream) {
+    (void)hipGetLastError();
+    const dim3 grid((unsigned)((n + 63) / 64)), block(256);
+    const uint16_t *in = static_cast<const uint16_t *>(full);
+    if (bf16) {
+        if (out_f32) hipLaunchKernelGGL((sum_over_batch_kernel<BF16, true>), grid, block, 0, stream, in, out, B, n, sb);
+        else hipLaunchKernelGGL((sum_over_batch_kernel<BF16, false>), grid, block, 0, stream, in, out, B, n, sb);
+    } else {
+        if (out_f32) hipLaunchKernelGGL((sum_over_batch_kernel<F16, true>), grid, block, 0, stream, in, out, B, n, sb);
+        else hipLaunchKernelGGL((sum_over_batch_kernel<F16, false>), grid, block, 0, stream, in, out, B, n, sb);
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream) {

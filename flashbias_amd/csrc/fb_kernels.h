@@ -42,6 +42,9 @@ hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_dkv(const BwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream);
+// out[j] = sum_b full[b * sb + j] for j < n; 16-bit elements in, the same type or fp32 out.
+hipError_t launch_sum_over_batch(const void *full, void *out, bool bf16, bool out_f32, int64_t B, int64_t n, int64_t sb,
+                                 hipStream_t stream);
 
 // Compute units of the current device (cached per device; 256 on MI355X).  The launchers pick
 // smaller query tiles when the larger ones would leave compute units without a workgroup.

@@ -216,17 +216,32 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     del keep
     dq_bias = dk_bias = None
     if q_bias is not None:
-        r = q_bias.shape[-1]  # the kernels may have run on zero-padded factors
-        dq_bias = _reduce_like(dqb_full[..., :r], q_bias)
-        dk_bias = _reduce_like(dkb_full[..., :r], k_bias)
+        dq_bias = _reduce_like(dqb_full, q_bias)
+        dk_bias = _reduce_like(dkb_full, k_bias)
     return dq, dk, dv, dq_bias, dk_bias
 
 
 def _reduce_like(full, ref):
-    """Sum a full (B, L, H, r) gradient over the dims in which ``ref`` was broadcast."""
-    dims = [i for i in (0, 2) if ref.shape[i] == 1 and full.shape[i] != 1]
+    """The gradient of ``ref`` from the full (B, L, H, r') gradient the kernels wrote: summed over
+    the dims in which ``ref`` was broadcast (in fp32; over the batch by the library's own
+    streaming kernel, bit-reproducibly), without the zero columns the kernels may have run with."""
+    rank = ref.shape[-1]
+    over_batch = ref.shape[0] == 1 and full.shape[0] != 1
+    over_heads = ref.shape[2] == 1 and full.shape[2] != 1
+    n = full[0].numel()
+    if over_batch and full.is_contiguous() and n % 8 == 0:
+        out = torch.empty((1,) + full.shape[1:], device=full.device, dtype=torch.float32 if over_heads else full.dtype)
+        batch = full.shape[0]
+
+        def call(_, stream):
+            return _lib.load().fb_sum_over_batch(full.data_ptr(), out.data_ptr(), _dtype_code(full.dtype),
+                                                 _dtype_code(out.dtype), batch, n, n, stream)
+        _launch(call, None, full.device)
+        full, over_batch = out, False
+    dims = [i for i, over in ((0, over_batch), (2, over_heads)) if over]
     if dims:
-        return full.sum(dim=dims, keepdim=True, dtype=torch.float32).to(ref.dtype)
+        full = full.sum(dim=dims, keepdim=True, dtype=torch.float32)
+    full = full[..., :rank].to(ref.dtype)
     return full if full.is_contiguous() else full.contiguous()
 
 

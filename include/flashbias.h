@@ -132,6 +132,16 @@ int fb_bwd(const fb_params *p, void *stream);
  * ordered on one stream are safe.  Nothing in the array has to be cleared between calls. */
 int fb_bwd_static(const fb_params *p, void *stream);
 
+/* The last step of the backward for factors that every batch entry shares: the kernels write such
+ * a factor's gradient in full (B, L, H, r) shape, and this sums it over the batch:
+ * out[j] = sum_b full[b * batch_stride + j] for j < n = L * H * r, accumulated in fp32 in a fixed
+ * order (bit-reproducible), written in the input dtype or (out_dtype = FB_F32) in fp32.  The
+ * reference has no such step: it hands the kernels the un-expanded tensors with expanded strides
+ * (flash_bias_triton.py:1227-1231), so every batch entry overwrites the same gradient rows.
+ * n and batch_stride must be multiples of 8 elements, full 16-byte aligned (FB_ERR_STRIDE else). */
+int fb_sum_over_batch(const void *full, void *out, int dtype, int out_dtype, int64_t B, int64_t n,
+                      int64_t batch_stride, void *stream);
+
 /* The backward in three phases, exported so that a harness can time them separately (call them in
  * this order: the two main kernels read what the preprocess wrote).
  *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400); fills the

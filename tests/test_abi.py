@@ -111,6 +111,22 @@ def test_check_rejects_backward(mutate, code):
         assert fn(p, None) == code
 
 
+@pytest.mark.parametrize("args,code", [
+    ((None, 0x1000, 1, 1, 4, 64, 64), -1),
+    ((0x1000, None, 1, 1, 4, 64, 64), -1),
+    ((0x1000, 0x2000, 2, 2, 4, 64, 64), -3),   # fp32 in
+    ((0x1000, 0x2000, 1, 0, 4, 64, 64), -3),   # bf16 in, fp16 out
+    ((0x1000, 0x2000, 1, 1, 0, 64, 64), -2),
+    ((0x1000, 0x2000, 1, 1, 4, 60, 64), -4),   # rows of 60 elements: not whole 16-byte chunks
+    ((0x1000, 0x2000, 1, 1, 4, 64, 32), -4),   # rows would overlap
+    ((0x1008, 0x2000, 1, 1, 4, 64, 64), -4),   # not 16-byte aligned
+])
+def test_sum_over_batch_rejects(args, code):
+    lib = _lib.load()
+    assert lib.fb_sum_over_batch(*args, None) == code  # rejected before any launch
+    assert lib.fb_last_error() != b""
+
+
 def test_null_params():
     lib = _lib.load()
     assert lib.fb_check(None, 0) == -1

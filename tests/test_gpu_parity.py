@@ -286,6 +286,32 @@ def test_causal_structure_is_exact(gpu_device):
         assert not torch.equal(o[:, cut:], o2[:, cut:]), cut
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,n,pitch", [(1, 8, 8), (37, 200, 200), (300, 64 * 5, 64 * 5 + 24), (4096, 1024, 1024)])
+def test_sum_over_batch_entry_point(gpu_device, dtype, B, n, pitch):
+    """fb_sum_over_batch against a float64 sum of the same 16-bit values: fp32 output to fp32
+    accuracy, 16-bit output to its rounding; the same bits on a second run."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _dtype_code, _stream
+    lib = _lib.load()
+    g = torch.Generator(device=gpu_device).manual_seed(B)
+    store = torch.randn(B, pitch, device=gpu_device, generator=g).to(dtype)
+    want = store[:, :n].double().sum(0)
+    code = _dtype_code(dtype)
+    outs = []
+    for out_dtype in (torch.float32, dtype, dtype):
+        out = torch.full((n + 8,), 7.0, device=gpu_device, dtype=out_dtype)
+        _lib.check_status(lib.fb_sum_over_batch(store.data_ptr(), out.data_ptr(), code, _dtype_code(out_dtype), B, n,
+                                                pitch, _stream()))
+        torch.cuda.synchronize()
+        assert (out[n:] == 7).all()  # nothing written past the row
+        outs.append(out[:n])
+    scale = max(want.abs().max().item(), 1.0)
+    assert (outs[0].double() - want).abs().max() <= 1e-5 * scale
+    assert (outs[1].double() - want).abs().max() <= 2.0 ** -8 * scale
+    assert torch.equal(outs[1], outs[2])
+
+
 def test_backward_reproducibility(gpu_device):
     """All five gradients are accumulated in registers in a fixed order (no atomics):
     bit-identical from run to run."""
