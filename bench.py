@@ -208,19 +208,29 @@ def _device_configs(dev):
     return cfgs
 
 
-def _sweep(dev, steps, warmup):
+def _sweep(dev, steps, warmup, only=None):
     import torch
     from flashbias_amd import workloads
     out = []
     for name, build in _device_configs(dev):
+        if only is not None and only not in name:
+            continue
         q, k, v, qb, kb, do, causal, r = build()
         B, L, H, d = q.shape
         leaves = [t.requires_grad_(True) for t in (q, k, v, qb, kb)]
         t_fwd, t_fb = _autograd_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
         f_fwd, f_bwd = workloads.flops(B, H, L, L, d, r, causal)
+        # algorithmic HBM bytes of a step: every input read once per pass, every output written once
+        # (forward: q k v factors -> o, lse; backward: q k v o dO factors lse -> dq dk dv and the factor
+        # gradients in the factors' own shapes)
+        size = lambda *ts: sum(t.numel() * t.element_size() for t in ts)
+        lse_bytes = 4 * B * H * L
+        hbm = (size(q, k, v, qb, kb) + size(q) + lse_bytes) + (size(q, k, v, q, do, qb, kb) + lse_bytes + size(q, k, v, qb, kb))
         out.append({"workload": name, "fwd_ms": round(t_fwd, 4), "fwd_bwd_ms": round(t_fb, 4),
                     "fwd_tflops": round(f_fwd / t_fwd / 1e9, 1), "fwd_bwd_tflops": round((f_fwd + f_bwd) / t_fb / 1e9, 1),
-                    "pct_of_bf16_mfma_peak": round(100 * (f_fwd + f_bwd) / t_fb / 1e9 / PEAK_BF16_TFLOPS, 2)})
+                    "pct_of_bf16_mfma_peak": round(100 * (f_fwd + f_bwd) / t_fb / 1e9 / PEAK_BF16_TFLOPS, 2),
+                    "hbm_algorithmic_gb": round(hbm / 1e9, 3), "hbm_gbs": round(hbm / t_fb / 1e6, 1),
+                    "pct_of_hbm_peak": round(100 * hbm / t_fb / 1e6 / PEAK_HBM_GBS, 2)})
         del q, k, v, qb, kb, do, leaves
         torch.cuda.empty_cache()
     return out
@@ -307,9 +317,9 @@ def headline(args):
         "bwd_ms": round(ms["fb_bwd"], 4),
         "kernel_ms": {k: round(v, 4) for k, v in ms.items()},
         "reference_formula_tflops": round(ref_fb / (ms_step * 1e-3) / 1e12, 2),
-        "roofline": {"kernel": "bwd_dkv_kernel (fb_bwd_dkv)", "bound": "mfma", "achieved": round(tflops_main, 2),
+        "roofline": {"kernel": "bwd_dkv_lean_kernel (fb_bwd_dkv)", "bound": "mfma", "achieved": round(tflops_main, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_main / PEAK_BF16_TFLOPS, 4),
-                     "traffic": _profiled_traffic("bwd_dkv_kernel")},
+                     "traffic": _profiled_traffic("bwd_dkv_lean_kernel")},
         "gate": gate,
     }
     del keep
@@ -439,6 +449,8 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the sweep, fp16, permuted-factors and provider timings (profiling runs)")
     ap.add_argument("--report", action="store_true", help="table over all named workloads")
+    ap.add_argument("--only", metavar="TEXT", help="time only the benchmark configurations whose name contains TEXT "
+                                                   "(as in the line's `sweep`; for profiling runs), print them as JSON")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="before the run, copy a 256 MiB buffer 3 times (a plain copy kernel of known size, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run)")
@@ -456,7 +468,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if args.report:
+    if args.only:
+        import torch
+        print(json.dumps({"sweep": _sweep(torch.device("cuda:0"), args.steps, args.warmup, args.only)}))
+    elif args.report:
         report(args)
     else:
         headline(args)

@@ -1,7 +1,7 @@
 // delta = rowsum(o * dout), the memory-bound first step of the backward pass.  The scratch
 // buffer receives what the two main kernels consume: -delta in its first B*H*Lq floats,
-// lse * log2(e) in the next B*H*Lq, and both again as one chunk of 16-bit parts per query
-// (stat_chunk, from stat_offset on) for the streamlined dk/dv kernel.
+// lse * log2(e) in the next B*H*Lq, and (where the streamlined dk/dv kernel will run) both again
+// as one chunk of 16-bit parts per query (stat_chunk, from stat_offset on).
 // Replaces _bwd_preprocess_do_o_dot of the reference (flash_bias/flash_bias_triton.py:358-400).
 // Also here: the sum over the batch of a full-shape factor gradient, the memory-bound last step
 // of the backward pass for factors that all batch entries share.
@@ -40,7 +40,7 @@ __global__ __launch_bounds__(256) void bwd_preprocess_kernel(const BwdArgs a) {
         const float l2 = a.lse[rix] * kLog2e;
         a.delta[rix] = -acc;
         a.delta[rows + rix] = l2;
-        reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[rix] = stat_chunk<T>(-acc, l2);
+        if (a.stat_chunks) reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[rix] = stat_chunk<T>(-acc, l2);
     }
 }
 
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void bwd_preprocess_chunks_kernel(const BwdArg
             const float l2 = a.lse[rix] * kLog2e;
             a.delta[rix] = -acc;
             a.delta[rows + rix] = l2;
-            reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[rix] = stat_chunk<T>(-acc, l2);
+            if (a.stat_chunks) reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[rix] = stat_chunk<T>(-acc, l2);
         }
     }
 }

@@ -613,7 +613,7 @@ static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
         // the streamlined kernel: same 128-key workgroups as the general one, and ahead of it at every
         // grid size (measured at B2 H4: 0.019 against 0.023 ms at L=1024, 0.063 against 0.082 at 4096,
         // 0.73 against 0.82 at 16384)
-        if (vec && dkv_lean_ok(a)) return launch_dkv_lean<T, NKR>(a, stream);
+        if (dkv_streamlined(a)) return launch_dkv_lean<T, NKR>(a, stream);
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lq)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);

@@ -396,16 +396,6 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     }
 }
 
-// Whether the streamlined kernel covers a call (the caller has already checked alignment and the
-// absence of a mask): head dim 32 exactly and rank 8 or none (the copies fill whole rows, there is
-// no zero padding of the channels).  With scale * log2(e) <= 1 the folded k cannot leave the 16-bit
-// range; a folded k_b that does sends its workgroup to the general kernel.
-inline bool dkv_lean_ok(const BwdArgs &a) {
-    const int64_t lim = (int64_t)1 << 24; // (32-bit tile row offsets in the copies)
-    return a.d == 32 && (a.r == 8 || a.r == 0) && a.scale > 1e-6f && a.scale * kLog2e <= 1.f && a.q.ss < lim &&
-           a.dout.ss < lim && (a.r == 0 || a.qb.ss < lim);
-}
-
 template <class T, int NKR>
 static hipError_t launch_dkv_lean(const BwdArgs &a0, hipStream_t stream) {
     typedef DkvLeanCfg<T, NKR> C;

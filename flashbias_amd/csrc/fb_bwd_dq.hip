@@ -256,7 +256,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
                 const int64_t rows = (int64_t)a.B * a.H * a.Lq;
                 a.delta[sidx] = nd;
                 a.delta[rows + sidx] = l2;
-                reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[sidx] = stat_chunk<T>(nd, l2);
+                if (a.stat_chunks) reinterpret_cast<u32x4_t *>(a.delta + stat_offset(rows))[sidx] = stat_chunk<T>(nd, l2);
             }
         } else {
             // the preprocess step left -delta and lse * log2(e) in the scratch buffer

@@ -35,7 +35,21 @@ struct BwdArgs {
     int ntiles_m; // query tiles per (batch, head), dq kernel
     int slots;    // workgroups of this launch that share a compute unit (priority turn-taking)
     int stats_here; // dq kernel: compute -delta and lse * log2(e) itself (and store them) instead of reading them
+    int stat_chunks; // writers of the scratch buffer: also store the statistics chunks (dkv_streamlined())
 };
+
+// Whether the backward of a call runs the streamlined dk/dv kernel (fb_bwd_dkv_lean.h), which is
+// also whether the writers of the scratch buffer (preprocess step, dq kernel) add the statistics
+// chunks it reads: aligned tensors, no mask, head dim 32 exactly and rank 8 or none (its copies
+// fill whole rows, there is no zero padding of the channels), row pitches that fit its 32-bit
+// offsets.  With scale * log2(e) <= 1 the folded k cannot leave the 16-bit range; a folded k_b
+// that does sends its workgroup to the general kernel.
+inline bool dkv_streamlined(const BwdArgs &a) {
+    const int64_t lim = (int64_t)1 << 24;
+    return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
+           (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.qb.ss < lim)) && a.q.ss < lim && a.dout.ss < lim &&
+           a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f;
+}
 
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.
 hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream);

@@ -147,7 +147,8 @@ int fb_sum_over_batch(const void *full, void *out, int dtype, int out_dtype, int
  *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400); fills the
  *                      scratch with -delta (first B*H*Lq floats), lse * log2(e) (next B*H*Lq) and, from the
  *                      next 16-byte boundary on, both once more per query row as three 16-bit parts each
- *                      (what the streamlined dk/dv kernel feeds to its MFMAs)
+ *                      (what the streamlined dk/dv kernel feeds to its MFMAs; written only for the calls
+ *                      that kernel takes: aligned, unmasked, head dim 32, rank 8 or 0)
  *   fb_bwd_dkv:        recompute P from lse; dk, dv, dk_bias, one workgroup per key tile
  *                      (_bwd_kernel / _bwd_kernel_one_col_block, :450-1097, minus dq)
  *   fb_bwd_dq:         recompute P from lse; dq, dq_bias, one workgroup per query tile
