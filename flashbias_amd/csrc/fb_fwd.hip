@@ -582,10 +582,12 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
         return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
     if constexpr (NKD == 2 && NKR <= 1 && NDV == 1) {
-        // the streamlined kernel has 256-query workgroups only: grids that fill the chip (see launch_fwd_vec)
+        // The streamlined kernel has 256-query workgroups only; its single wave per SIMD still beats
+        // the general kernel's smaller tiles down to a quarter-filled chip (measured at B2 H4: 0.122
+        // against 0.173 ms at L=8192, 0.054 against 0.059 at 4096, 0.029 against 0.030 at 2048; at
+        // L=1024, 32 workgroups, 0.0175 against 0.0169).
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (vec && fwd_lean_ok(a) && wgs >= (int64_t)2 * num_cus())
-            return launch_fwd_lean<T, NKR>(a, stream);
+        if (vec && fwd_lean_ok(a) && 4 * wgs >= num_cus()) return launch_fwd_lean<T, NKR>(a, stream);
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);
