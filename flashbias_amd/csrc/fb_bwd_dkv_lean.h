@@ -49,19 +49,6 @@ __device__ __attribute__((noinline)) void dkv_lean_retry() {
     bwd_dkv_body<T, typename C::General>(a);
 }
 
-// acc += A B with the accumulator tied to the result register block (the compiler's own choice
-// often is a second block and a copy).  The compiler does not see an MFMA here, so the caller owes
-// the two wait states between a VALU write of a or b and this instruction (the block step below
-// converts P and dS at least one slot before their use) and the wait for the last result before
-// anything but another such MFMA reads acc.
-template <class T>
-__device__ __forceinline__ void mfma_into(f32x16_t &acc, const u32x4_t &a, const u32x4_t &b) {
-    if constexpr (std::is_same<T, BF16>::value)
-        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-    else
-        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
-}
-
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkv_lean_kernel(const BwdArgs a) {
     constexpr int NKR = C::NKR;

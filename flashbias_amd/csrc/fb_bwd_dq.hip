@@ -520,6 +520,10 @@ static hipError_t launch_dq_vec(const BwdArgs &a, hipStream_t stream) {
     return launch_dq_qb<T, NKD, NKR, VEC, MASK, true, FOLD>(a, stream);
 }
 
+} // namespace fb
+#include "fb_bwd_dq_lean.h"
+namespace fb {
+
 template <class T, int NKD, int NKR>
 static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
     // the direct loader keeps the byte distance between two tiles' rows in 32 bits
@@ -529,6 +533,9 @@ static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
                      (a.r == 0 || a.kb.ss < lim) && (!a.stats_here || a.o.vec_ok);
     if (a.mask.type)
         return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
+    if constexpr (NKD == 2 && NKR <= 1) {
+        if (dq_streamlined(a)) return launch_dq_lean<T, NKR>(a, stream);
+    }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_dq_vec<T, NKD, NKR, true, false, true>(a, stream);
     }

@@ -51,6 +51,14 @@ inline bool dkv_streamlined(const BwdArgs &a) {
            a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f;
 }
 
+// The same for the streamlined dq kernel (fb_bwd_dq_lean.h), which streams K, K_b and V.
+inline bool dq_streamlined(const BwdArgs &a) {
+    const int64_t lim = (int64_t)1 << 24;
+    return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
+           (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.kb.ss < lim)) && a.k.ss < lim && a.v.ss < lim &&
+           (!a.stats_here || a.o.vec_ok) && a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f;
+}
+
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.
 hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream);

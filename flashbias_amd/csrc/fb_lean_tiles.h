@@ -12,6 +12,8 @@
 // region, every lane fetching the chunk that belongs at its position: all lanes on, one tensor per
 // instruction, nothing to set up but the scalar base and m0.
 #pragma once
+#include <type_traits>
+
 #include "fb_device.h"
 
 namespace fb {
@@ -140,5 +142,18 @@ struct LeanCopy2 {
     // copy instructions this wave issues per tile
     __device__ __forceinline__ static int count(int wave) { return (ROWS < 128 && wave >= ROWS / 32) ? 0 : 1; }
 };
+
+// acc += A B with the accumulator tied to the result register block (the compiler's own choice
+// often is a second block and a copy).  The compiler does not see an MFMA here, so the caller owes
+// the two wait states between a VALU write of a or b and this instruction (the block step below
+// converts P and dS at least one slot before their use) and the wait for the last result before
+// anything but another such MFMA reads acc.
+template <class T>
+__device__ __forceinline__ void mfma_into(f32x16_t &acc, const u32x4_t &a, const u32x4_t &b) {
+    if constexpr (std::is_same<T, BF16>::value)
+        asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+    else
+        asm("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
 
 } // namespace fb
