@@ -44,8 +44,8 @@ struct DkvLeanCfg {
 };
 
 template <class T, class C>
-__device__ __attribute__((noinline)) void dkv_lean_retry() {
-    const BwdArgs a = *(const BwdArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+__device__ __attribute__((noinline)) void dkv_lean_retry(const void *kernargs) {
+    const BwdArgs a = uniform_kernargs<BwdArgs>(kernargs);
     bwd_dkv_body<T, typename C::General>(a);
 }
 
@@ -94,7 +94,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         }
     }
     if (__syncthreads_or(bad)) {
-        dkv_lean_retry<T, C>();
+        dkv_lean_retry<T, C>((const void *)__builtin_amdgcn_kernarg_segment_ptr());
         return;
     }
     // ones against the parts of -lse * log2(e) (k-slots 0..2) and of -delta (k-slots 3..5)

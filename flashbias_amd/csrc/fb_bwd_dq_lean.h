@@ -40,8 +40,8 @@ struct DqLeanCfg {
 };
 
 template <class T, class C>
-__device__ __attribute__((noinline)) void dq_lean_retry() {
-    const BwdArgs a = *(const BwdArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+__device__ __attribute__((noinline)) void dq_lean_retry(const void *kernargs) {
+    const BwdArgs a = uniform_kernargs<BwdArgs>(kernargs);
     bwd_dq_body<T, typename C::General>(a);
 }
 
@@ -90,7 +90,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         }
     }
     if (__syncthreads_or(bad)) {
-        dq_lean_retry<T, C>();
+        dq_lean_retry<T, C>((const void *)__builtin_amdgcn_kernarg_segment_ptr());
         return;
     }
     // -lse * log2(e) and -delta of this lane's query

@@ -582,12 +582,11 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
         return vec ? launch_fwd_vec<T, NKD, NKR, NDV, true, true>(a, stream)
                    : launch_fwd_vec<T, NKD, NKR, NDV, false, true>(a, stream);
     if constexpr (NKD == 2 && NKR <= 1 && NDV == 1) {
-        // The streamlined kernel has 256-query workgroups only; its single wave per SIMD still beats
-        // the general kernel's smaller tiles down to a quarter-filled chip (measured at B2 H4: 0.122
-        // against 0.173 ms at L=8192, 0.054 against 0.059 at 4096, 0.029 against 0.030 at 2048; at
-        // L=1024, 32 workgroups, 0.0175 against 0.0169).
+        // The streamlined kernel: 256-query workgroups (two query blocks per wave) where they give every
+        // SIMD of the chip a wave, 128-query workgroups (one block per wave) below that.
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (vec && fwd_lean_ok(a) && 4 * wgs >= num_cus()) return launch_fwd_lean<T, NKR>(a, stream);
+        if (vec && fwd_lean_ok(a))
+            return wgs >= num_cus() ? launch_fwd_lean<T, NKR, 2>(a, stream) : launch_fwd_lean<T, NKR, 1>(a, stream);
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);

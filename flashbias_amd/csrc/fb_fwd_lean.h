@@ -11,7 +11,8 @@
 //   * m is fixed per query for the whole key loop: the maximum over the first key block.  No
 //     running maximum, no rescale.  p = 2^(s - m) is then not bounded by 1, which costs nothing in
 //     floating point as long as nothing overflows; the row sum tells: a workgroup in which a row
-//     sum leaves [2^-60, 2^60] (or is NaN) throws its work away and runs the general algorithm
+//     sum leaves [2^-60, 2^60] (fp16, whose P must fit 16 bits: [2^-7, 60000]; or is NaN) throws
+//     its work away and runs the general algorithm
 //     (fwd_body: unscaled operands, the scale applied to the fp32 q k^T accumulator as in the
 //     reference, flash_bias_triton.py:246-256, running maximum).  That is the safety net for
 //     adversarial inputs and for 16-bit overflow of the scaled operands, not something the benchmark
@@ -39,34 +40,38 @@ namespace fb {
 // and the transposing 8-byte reads of V, then touch every bank once.  A copy instruction fills 64
 // consecutive positions (8 lines) of one region, every lane fetching the chunk that belongs at its
 // position: all lanes on, one tensor per instruction, nothing but a scalar base and m0 to set up.
-template <class T, int NKR_>
+// QB_: query blocks (of 32) per wave.  Two where the grid fills the chip (every key / value fragment
+// read from LDS then feeds two blocks); one on small grids, which doubles the number of waves.
+template <class T, int NKR_, int QB_ = 2>
 struct FwdLeanCfg {
-    static constexpr int NKD = 2, NKR = NKR_, NK = NKD + NKR_;
+    static constexpr int NKD = 2, NKR = NKR_, NK = NKD + NKR_, QB = QB_;
     static_assert(NKR_ <= 1, "rank <= 8");
-    static constexpr int NWAVES = 4, NTHREADS = 256, BM = 256, BN = 128, KB = BN / 32;
+    static_assert(QB_ == 1 || QB_ == 2, "");
+    static constexpr int NWAVES = 4, NTHREADS = 256, BM = 128 * QB_, BN = 128, KB = BN / 32;
     static constexpr int K_BYTES = BN * 64, B_BYTES = NKR_ ? BN * 32 : 0, V_BYTES = BN * 64;
     static constexpr int B_OFF = K_BYTES, V_OFF = K_BYTES + B_BYTES, STAGE_BYTES = V_OFF + V_BYTES;
     static constexpr int NSTAGE = 3;
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES;
     // copy instructions per wave and tile: 2 of K (16 rows each), 2 of V, 1 of K_b (32 rows)
     static constexpr int NDMA = 4 + (NKR_ ? 1 : 0);
-    // the general configuration a workgroup falls back to (same 256 queries per workgroup)
-    typedef FwdCfg<T, 2, NKR_, 1, true, false, true, false> General;
+    // the general configuration a workgroup falls back to (same queries per workgroup)
+    typedef FwdCfg<T, 2, NKR_, 1, true, false, QB_ == 2, false> General;
     static_assert(General::BM == BM && General::LDS_BYTES <= LDS_BYTES, "");
 };
 
-// Out of line, and reading the kernel arguments from the kernel-argument segment itself: the
-// streamlined kernel keeps its own copy in scalar registers, and neither its register allocation
-// nor the uniformity of its control flow is disturbed by this path.
+// Out of line, and reading the kernel arguments from the kernel-argument segment, whose address
+// the kernel hands over (the intrinsic that returns it is only meaningful in the kernel itself: in
+// a function it yields null): the streamlined kernel keeps its own copy in scalar registers, and
+// neither its register allocation nor the uniformity of its control flow is disturbed by this path.
 template <class T, class C>
-__device__ __attribute__((noinline)) void fwd_lean_retry() {
-    const FwdArgs a = *(const FwdArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+__device__ __attribute__((noinline)) void fwd_lean_retry(const void *kernargs) {
+    const FwdArgs a = uniform_kernargs<FwdArgs>(kernargs);
     fwd_body<T, typename C::General>(a);
 }
 
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void fwd_lean_kernel(const FwdArgs a) {
-    constexpr int NK = C::NK, NKD = C::NKD, NKR = C::NKR;
+    constexpr int NK = C::NK, NKD = C::NKD, NKR = C::NKR, QB = C::QB;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int tile_m = work % a.ntiles_m;
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
-    const int wq0 = m0 + wave * 64; // first query of this wave
+    const int wq0 = m0 + wave * (32 * QB); // first query of this wave
 
     const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
     const uint8_t *kptr = reinterpret_cast<const uint8_t *>(a.k.ptr + b * a.k.sb + h * a.k.sh);
@@ -93,9 +98,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 
     // ---- resident query operands, in exponent-of-2 units (rows past the end are zero)
     const float cq = a.scale * kLog2e;
-    u32x4_t qr[2][NKD], qbr[2][NKR > 0 ? NKR : 1];
+    u32x4_t qr[QB][NKD], qbr[QB][NKR > 0 ? NKR : 1];
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < QB; ++qb) {
         const int query = wq0 + 32 * qb + c;
 #pragma unroll
         for (int t = 0; t < NKD; ++t)
@@ -197,9 +202,17 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     };
 
     // One reference point per lane serves both of its queries (any value near a row's maximum
-    // does): the larger of the two estimates, in all 16 registers of one block.
-    f32x16_t acc_o[2], minit;
-    float l_run[2], m2;
+    // does): the larger of the two estimates, in all 16 registers of one block.  P = 2^(s - m) goes
+    // to the PV MFMA as a 16-bit value: bf16 has fp32's range, but fp16 ends at 65504 and loses
+    // precision below 2^-14, so for fp16 the reference point sits 6 powers of two above the
+    // estimate (22 of head room above it, the estimate's own key at 2^-6) and the row sum, which
+    // bounds every P of the row from above, has to stay within [2^-7, 60000] instead of
+    // [2^-60, 2^60]: outside, the workgroup takes the general algorithm.
+    constexpr bool kHalf = std::is_same<T, F16>::value;
+    constexpr float kShift = kHalf ? 6.f : 0.f;
+    constexpr float kLmin = kHalf ? 0x1p-7f : 0x1p-60f, kLmax = kHalf ? 60000.f : 0x1p60f;
+    f32x16_t acc_o[QB], minit;
+    float l_run[QB], m2;
     // p = 2^s for the 16 scores of a block, row sums, O^T += V^T P^T
     auto softmax_pv = [&](const f32x16_t &s, const u32x4_t (&f)[2], int qb) {
 #pragma unroll
@@ -241,7 +254,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         float mx = -INFINITY;
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
+        for (int qb = 0; qb < QB; ++qb) {
             f32x16_t s = scores(ka, qb, zero16);
             hide(s, 0);
 #pragma unroll
@@ -250,7 +263,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc_o[qb][v] = 0.f;
         }
-        m2 = half_wave_max(mx);
+        m2 = half_wave_max(mx) + kShift;
 #pragma unroll
         for (int v = 0; v < 16; ++v) minit[v] = -m2;
     }
@@ -267,19 +280,21 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         f32x16_t s_cur, s_nxt;
         read_ka(ka, STG, 0);
         s_cur = scores(ka, 0, minit);
-        // one key block: both query blocks against fragments `cur`, the fragments of the next key
-        // block arrive in `nxt` meanwhile
+        // one key block: every query block of the wave against fragments `cur`, the fragments of
+        // the next key block arrive in `nxt` meanwhile
         auto key_block = [&](u32x4_t (&cur)[NK], u32x4_t (&nxt)[NK], int kb, bool hidden_pairs) {
             if (kb + 1 < C::KB) read_ka(nxt, STG, kb + 1);
             read_va(va, STG, kb);
-            s_nxt = scores(cur, 1, minit);
-            if (hidden_pairs) hide(s_cur, n0 + 32 * kb);
-            softmax_pv(s_cur, va, 0);
-            s_cur = s_nxt;
-            interleave();
+            if constexpr (QB == 2) {
+                s_nxt = scores(cur, 1, minit);
+                if (hidden_pairs) hide(s_cur, n0 + 32 * kb);
+                softmax_pv(s_cur, va, 0);
+                s_cur = s_nxt;
+                interleave();
+            }
             if (kb + 1 < C::KB) s_nxt = scores(nxt, 0, minit);
             if (hidden_pairs) hide(s_cur, n0 + 32 * kb);
-            softmax_pv(s_cur, va, 1);
+            softmax_pv(s_cur, va, QB - 1);
             s_cur = s_nxt;
             interleave();
         };
@@ -313,20 +328,20 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     // ---- did every row sum stay in range?  (The decision is the workgroup's: the fallback needs all waves.)
     bool bad = false;
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < QB; ++qb) {
         const float l = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
         l_run[qb] = l;
-        if (wq0 + 32 * qb + c < a.Lq && !(l >= 0x1p-60f && l <= 0x1p60f)) bad = true;
+        if (wq0 + 32 * qb + c < a.Lq && !(l >= kLmin && l <= kLmax)) bad = true;
     }
     if (__syncthreads_or(bad)) {
-        fwd_lean_retry<T, C>();
+        fwd_lean_retry<T, C>((const void *)__builtin_amdgcn_kernarg_segment_ptr());
         return;
     }
 
     // ---- epilogue: o = acc / l, lse = (m + log2 l) ln 2
     uint16_t *obase = const_cast<uint16_t *>(a.o.ptr) + b * a.o.sb + h * a.o.sh;
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
+    for (int qb = 0; qb < QB; ++qb) {
         const int query = wq0 + 32 * qb + c;
         const float l = l_run[qb];
         const float inv = 1.f / l;
@@ -347,9 +362,11 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 
 // Whether the streamlined kernel covers a call (the caller has already checked alignment and the
 // absence of a mask): head dim 32 exactly and rank 8 or none (the copies fill whole rows, there is
-// no zero padding of the channels); the factors then fit the hi + lo layout of one bias step.  The bounds
-// on the scale keep the folded operands away from the ends of fp32's range; what a 16-bit type
-// cannot hold after the scaling ends up as inf / NaN row sums, which take the fallback.
+// no zero padding of the channels); the factors then fit the hi + lo layout of one bias step.  The
+// folded query operand is rounded to 16 bits once more, which puts a relative 2^-9 on every q k
+// product: harmless for logits of order one, visible in o for logits in the tens, hence the bound
+// scale * log2(e) <= 1 (which also keeps the folded operand inside the 16-bit range; what a folded
+// factor cannot hold ends up as inf / NaN row sums, which take the fallback).
 // Not for causal calls nor for fewer than 128 keys: with a reference point that is not the row's
 // own maximum the largest P of a row is not exactly 1, so a row that sees one or two keys comes
 // out an ulp off v (the general kernel returns it exactly), and the reference point of a query
@@ -357,13 +374,13 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 // independence of o[i] from keys j > i.
 inline bool fwd_lean_ok(const FwdArgs &a) {
     const int64_t lim = (int64_t)1 << 24; // (32-bit tile row offsets in the copies)
-    return a.d == 32 && (a.r == 8 || a.r == 0) && !a.causal && a.Lk >= 128 && a.scale > 1e-6f && a.scale < 1e6f &&
+    return a.d == 32 && (a.r == 8 || a.r == 0) && !a.causal && a.Lk >= 128 && a.scale > 1e-6f && a.scale * kLog2e <= 1.f &&
            a.k.ss < lim && a.v.ss < lim && (a.r == 0 || a.kb.ss < lim);
 }
 
-template <class T, int NKR>
+template <class T, int NKR, int QB>
 static hipError_t launch_fwd_lean(const FwdArgs &a0, hipStream_t stream) {
-    typedef FwdLeanCfg<T, NKR> C;
+    typedef FwdLeanCfg<T, NKR, QB> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_lean_kernel<T, C>;

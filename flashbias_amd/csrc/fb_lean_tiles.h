@@ -143,6 +143,26 @@ struct LeanCopy2 {
     __device__ __forceinline__ static int count(int wave) { return (ROWS < 128 && wave >= ROWS / 32) ? 0 : 1; }
 };
 
+// The kernel arguments as a function called by the kernel may read them: a function's pointer
+// argument arrives in vector registers, which would make every value loaded through it look
+// divergent (vector loads, no scalar operands for the copy instructions); made wave-uniform again
+// and typed as constant memory it is read with scalar loads like the kernel's own copy.
+template <class A>
+__device__ __forceinline__ A uniform_kernargs(const void *p) {
+    static_assert(sizeof(A) % 4 == 0, "");
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint64_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint64_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    const __attribute__((address_space(4))) uint32_t *w = (const __attribute__((address_space(4))) uint32_t *)((hi << 32) | lo);
+    union {
+        A a;
+        uint32_t u[sizeof(A) / 4];
+    } x;
+#pragma unroll
+    for (unsigned i = 0; i < sizeof(A) / 4; ++i) x.u[i] = w[i];
+    return x.a;
+}
+
 // acc += A B with the accumulator tied to the result register block (the compiler's own choice
 // often is a second block and a copy).  The compiler does not see an MFMA here, so the caller owes
 // the two wait states between a VALU write of a or b and this instruction (the block step below

@@ -407,6 +407,29 @@ def test_streamlined_kernels(gpu_device, dtype, r, causal):
     _case(gpu_device, B, Lq, Lk, H, 32, r, dtype, causal, seed=14)
 
 
+@pytest.mark.parametrize("which", ["q_bias", "k_bias", "logits"])
+def test_streamlined_kernels_fall_back(gpu_device, which):
+    """Inputs the streamlined kernels cannot take make their workgroups run the general algorithm
+    instead: an fp16 factor entry that overflows once log2(e) is folded into it (60000, facing a zero
+    column of the other factor, so the bias itself is unchanged: q_bias for the forward and dq
+    kernels, k_bias for dk/dv), and logits so peaked that P = 2^(s - m) with the fixed reference
+    point leaves fp16's range (unscaled N(0,1) factors of rank 8, as in the reference's own
+    correctness script, at a length where some row sums exceed the limit)."""
+    B, L, H, d, r = 2, 640, 2, 32, 8
+    q, k, v, qb, kb, do = make_inputs(B, L, L, H, d, r, torch.float16, seed=15)
+    if which == "logits":
+        g = torch.Generator().manual_seed(16)
+        qb, kb = [torch.randn(B, L, H, r, generator=g).half() * 1.5 for _ in range(2)]
+    else:
+        big, zero = (qb, kb) if which == "q_bias" else (kb, qb)
+        zero[..., 3] = 0
+        big[:, ::7, :, 3] = 60000.0
+        do = (do.float() * 0.03).half()  # (keeps the gradient of the zero column, ~ 60000 dS, inside fp16)
+    ref = oracle(q, k, v, qb, kb, None, False, None, do)
+    got = run_gpu(flash_bias_func, q, k, v, qb, kb, None, False, None, do, gpu_device)
+    _gate(got, ref, torch.float16)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("offset", [0, 1])
 def test_matrix_mask_alignment(gpu_device, dtype, offset):
