@@ -278,4 +278,42 @@ class FlashBiasFunc(torch.autograd.Function):
         return dq, dk, dv, dq_bias, dk_bias, None, None, None
 
 
-flash_bias_func = FlashBiasFunc.apply
+_ext = False  # the C++ autograd function: False = not looked for yet, None = not built
+
+
+def _extension():
+    """flashbias_amd/_fb_torch.so (csrc/fb_torch.cpp): the autograd function of the operator in C++,
+    over the same C ABI.  None when it has not been built; the Python FlashBiasFunc then serves."""
+    global _ext
+    if _ext is False:
+        try:
+            from . import _fb_torch
+            _lib.load()
+            _ext = _fb_torch
+        except ImportError:
+            _ext = None
+    return _ext
+
+
+def flash_bias_func(q, k, v, q_bias=None, k_bias=None, mask=None, causal=False, softmax_scale=None):
+    """``FlashBiasFunc.apply`` of the reference (flash_bias/flash_bias_triton.py:1405): same positional
+    arguments and defaults.  Runs the autograd function in C++ when that extension is built (the
+    same checks, allocations and launches without the interpreter: a forward + backward costs the
+    host about half as much, which is what sequence lengths up to a few thousand are bound by),
+    else the Python FlashBiasFunc above.  The rare preparations (a large vector mask folded into the
+    factors, a rank padded to a multiple of 8) are ordinary differentiable tensor operations here,
+    so their gradients come from autograd."""
+    ext = _extension()
+    if ext is None:
+        return FlashBiasFunc.apply(q, k, v, q_bias, k_bias, mask, causal, softmax_scale)
+    # the launcher's assertions (:1100-1143), as assertions
+    assert q.dim() == 4 and k.dim() == 4 and k.shape[0] == q.shape[0] and k.shape[2:] == q.shape[2:] and v.shape == k.shape
+    assert q.shape[-1] <= 128, "FlashBias only supports head dimensions up to 128"
+    assert q.dtype == k.dtype == v.dtype, "All tensors must have the same type"
+    assert q.dtype in (torch.float16, torch.bfloat16), "Only support fp16 and bf16"
+    assert q.is_cuda and k.is_cuda and v.is_cuda
+    if (q_bias is not None and q_bias.shape[-1] % 8) or (mask is not None and mask.dim() == 4 and mask.shape[2] == 1):
+        if q_bias is not None:
+            q, k, v, q_bias, k_bias = [_last_dim_contiguous(x) for x in (q, k, v, q_bias, k_bias)]
+        q_bias, k_bias, mask = _prepare_factors(q, k, q_bias, k_bias, mask)
+    return ext.flash_bias(q, k, v, q_bias, k_bias, mask, bool(causal), float(softmax_scale or 0.0))

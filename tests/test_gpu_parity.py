@@ -312,6 +312,37 @@ def test_sum_over_batch_entry_point(gpu_device, dtype, B, n, pitch):
     assert torch.equal(outs[1], outs[2])
 
 
+@pytest.mark.parametrize("case", ["plain", "rank5_shared_by_heads", "shared_by_batch_vector_mask", "matrix_mask_no_factors"])
+def test_cpp_and_python_autograd_functions_agree(gpu_device, case):
+    """flash_bias_func runs the autograd function in C++ (flashbias_amd/_fb_torch.so) when that is
+    built; FlashBiasFunc is the same in Python.  Same library calls, so the same bits, for the output
+    and every gradient."""
+    from flashbias_amd import FlashBiasFunc, interface
+    assert interface._extension() is not None, "flashbias_amd/_fb_torch.so is not built"
+    dev, dt = gpu_device, torch.bfloat16
+    B, L, H, d = 3, 200, 4, 32
+    g = torch.Generator().manual_seed(21)
+    q, k, v, do = [torch.randn(B, L, H, d, generator=g).to(dt).to(dev) for _ in range(4)]
+    qb = kb = mask = None
+    if case == "plain":
+        qb, kb = [(torch.randn(B, L, H, 8, generator=g) / 3).to(dt).to(dev) for _ in range(2)]
+    elif case == "rank5_shared_by_heads":
+        qb, kb = [(torch.randn(B, L, 1, 5, generator=g) / 2).to(dt).to(dev) for _ in range(2)]
+    elif case == "shared_by_batch_vector_mask":
+        qb, kb = [(torch.randn(1, L, H, 16, generator=g) / 4).to(dt).to(dev) for _ in range(2)]
+        mask = torch.zeros(B, 1, 1, L, dtype=dt).masked_fill(torch.rand(B, 1, 1, L, generator=g) < 0.2, float("-inf")).to(dev)
+    else:
+        mask = torch.randn(1, H, L, L, generator=g).to(dt).to(dev)
+    outs = []
+    for fn in (flash_bias_func, FlashBiasFunc.apply):
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, v)] + ([t.clone().requires_grad_(True) for t in (qb, kb)] if qb is not None else [])
+        bias = leaves[3:] if qb is not None else [None, None]
+        o = fn(leaves[0], leaves[1], leaves[2], bias[0], bias[1], mask, case == "plain", None)
+        outs.append([o.detach()] + list(torch.autograd.grad(o, leaves, do)))
+    for a, b in zip(*outs):
+        assert a.shape == b.shape and torch.equal(a, b)
+
+
 def test_backward_reproducibility(gpu_device):
     """All five gradients are accumulated in registers in a fixed order (no atomics):
     bit-identical from run to run."""
