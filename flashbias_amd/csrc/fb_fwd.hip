@@ -585,7 +585,10 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
         // The streamlined kernel: 256-query workgroups (two query blocks per wave) where they give every
         // SIMD of the chip a wave, 128-query workgroups (one block per wave) below that.
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (vec && fwd_lean_ok(a))
+        // On grids that fill the chip a loop of at least 512 keys pays for the kernel's pipeline (4096 x 16
+        // windows, general against streamlined: 1.91 against 2.82 ms at 128 keys, 1.79 against 1.88 at 256,
+        // 1.38 against 1.21 at 512); small grids take it at every length.
+        if (vec && fwd_lean_ok(a) && (a.Lk >= 512 || small_grid(a.B, a.H, a.Lq)))
             return wgs >= num_cus() ? launch_fwd_lean<T, NKR, 2>(a, stream) : launch_fwd_lean<T, NKR, 1>(a, stream);
     }
     if constexpr (NKR <= 2) {

@@ -38,27 +38,6 @@ struct BwdArgs {
     int stat_chunks; // writers of the scratch buffer: also store the statistics chunks (dkv_streamlined())
 };
 
-// Whether the backward of a call runs the streamlined dk/dv kernel (fb_bwd_dkv_lean.h), which is
-// also whether the writers of the scratch buffer (preprocess step, dq kernel) add the statistics
-// chunks it reads: aligned tensors, no mask, head dim 32 exactly and rank 8 or none (its copies
-// fill whole rows, there is no zero padding of the channels), row pitches that fit its 32-bit
-// offsets.  With scale * log2(e) <= 1 the folded k cannot leave the 16-bit range; a folded k_b
-// that does sends its workgroup to the general kernel.
-inline bool dkv_streamlined(const BwdArgs &a) {
-    const int64_t lim = (int64_t)1 << 24;
-    return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
-           (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.qb.ss < lim)) && a.q.ss < lim && a.dout.ss < lim &&
-           a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f;
-}
-
-// The same for the streamlined dq kernel (fb_bwd_dq_lean.h), which streams K, K_b and V.
-inline bool dq_streamlined(const BwdArgs &a) {
-    const int64_t lim = (int64_t)1 << 24;
-    return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
-           (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.kb.ss < lim)) && a.k.ss < lim && a.v.ss < lim &&
-           (!a.stats_here || a.o.vec_ok) && a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f;
-}
-
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.
 hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream);
@@ -80,6 +59,39 @@ inline int num_cus() {
         cached[dev].store(n, std::memory_order_relaxed); // (concurrent first calls store the same value)
     }
     return n;
+}
+
+// A grid that leaves the chip under-filled even at the general kernels' occupancy: fewer than two
+// 128-row workgroups per compute unit.
+inline bool small_grid(int B, int H, int L) { return (int64_t)B * H * ((L + 127) / 128) < 2 * (int64_t)num_cus(); }
+
+// Whether the backward of a call runs the streamlined dk/dv kernel (fb_bwd_dkv_lean.h), which is
+// also whether the writers of the scratch buffer (preprocess step, dq kernel) add the statistics
+// chunks it reads: aligned tensors, no mask, head dim 32 exactly and rank 8 or none (its copies
+// fill whole rows, there is no zero padding of the channels), row pitches that fit its 32-bit
+// offsets.  With scale * log2(e) <= 1 the folded k cannot leave the 16-bit range; a folded k_b
+// that does sends its workgroup to the general kernel.  And a loop long enough to pay for the
+// kernel's six-stage pipeline: on grids that fill the chip the general kernel's three waves per SIMD
+// hide a short loop's latencies better (4096 x 16 windows, general against streamlined: 2.61 against
+// 3.09 ms at 256 queries, 2.05 against 2.18 at 512, 0.457 against 0.442 at 1024 with B64 H16); on
+// small grids the streamlined kernel is ahead at every length measured (B2 H4 from L=1024).
+inline bool dkv_streamlined(const BwdArgs &a) {
+    const int64_t lim = (int64_t)1 << 24;
+    return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
+           (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.qb.ss < lim)) && a.q.ss < lim && a.dout.ss < lim &&
+           a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f && (a.Lq >= 1024 || small_grid(a.B, a.H, a.Lk));
+}
+
+// The same for the streamlined dq kernel (fb_bwd_dq_lean.h), which streams K, K_b and V (general
+// against streamlined on grids that fill the chip: 2.10 against 2.86 ms at 4096 x 16 windows of 256
+// keys, 1.61 against 1.84 at 512, 0.352 against 0.371 at 1024 with B64 H16, 0.150 against 0.117 at
+// 2048 causal).
+inline bool dq_streamlined(const BwdArgs &a) {
+    const int64_t lim = (int64_t)1 << 24;
+    return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
+           (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.kb.ss < lim)) && a.k.ss < lim && a.v.ss < lim &&
+           (!a.stats_here || a.o.vec_ok) && a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f &&
+           (a.Lk >= 2048 || small_grid(a.B, a.H, a.Lq));
 }
 
 // What a launcher remembers about one kernel instantiation (one static object per instantiation;
