@@ -504,12 +504,14 @@ static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
 
 // 256-query workgroups (two blocks per wave) once every compute unit has two of them (four under
 // a causal mask: B1 H50 d32 at L=4096 is 11 % faster with the small ones, equal at L=8192, 3 %
-// slower at L=16384), 128-query workgroups below that: as in the forward launcher.
+// slower at L=16384), 128-query workgroups below that and for short sequences whose last 256-query
+// workgroup would be half empty (8192 x 16 windows of 128 tokens: 2.59 -> 1.76 ms): as in the forward
+// launcher.
 template <class T, int NKD, int NKR, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_dq_vec(const BwdArgs &a, hipStream_t stream) {
     if constexpr (DqCfg<T, NKD, NKR, VEC, MASK, true>::QBLK == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (wgs < (int64_t)(a.causal ? 4 : 2) * num_cus())
+        if (wgs < (int64_t)(a.causal ? 4 : 2) * num_cus() || half_empty_256(a.Lq))
             return launch_dq_qb<T, NKD, NKR, VEC, MASK, false, FOLD>(a, stream);
     }
     // head dims above 64, aligned, unmasked, rank <= 32: 32-key tiles fit two workgroups per CU

@@ -560,12 +560,13 @@ static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
 // (measured: 35 % faster at a quarter of that grid, 10 % slower at twice it).  Under a causal mask
 // the workgroups differ in length and the short ones leave the chip part empty towards the end:
 // the small workgroups stay ahead up to seven per compute unit (B1 H50 d32: 13 % faster at
-// L=4096, 5 % at L=8192, equal at L=16384).
+// L=4096, 5 % at L=8192, equal at L=16384).  Short sequences whose last 256-query workgroup would be half
+// empty also take the small ones (8192 x 16 windows of 128 tokens: 1.94 -> 1.41 ms).
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_fwd_vec(const FwdArgs &a, hipStream_t stream) {
     if constexpr (FwdCfg<T, NKD, NKR, NDV, VEC, MASK, true>::QB == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (wgs < (int64_t)(a.causal ? 7 : 2) * num_cus())
+        if (wgs < (int64_t)(a.causal ? 7 : 2) * num_cus() || half_empty_256(a.Lq))
             return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, false, FOLD>(a, stream);
     }
     return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, true, FOLD>(a, stream);
@@ -589,7 +590,8 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
         // windows, general against streamlined: 1.91 against 2.82 ms at 128 keys, 1.79 against 1.88 at 256,
         // 1.38 against 1.21 at 512); small grids take it at every length.
         if (vec && fwd_lean_ok(a) && (a.Lk >= 512 || small_grid(a.B, a.H, a.Lq)))
-            return wgs >= num_cus() ? launch_fwd_lean<T, NKR, 2>(a, stream) : launch_fwd_lean<T, NKR, 1>(a, stream);
+            return wgs >= num_cus() && !half_empty_256(a.Lq) ? launch_fwd_lean<T, NKR, 2>(a, stream)
+                                                             : launch_fwd_lean<T, NKR, 1>(a, stream);
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);

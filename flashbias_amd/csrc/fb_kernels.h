@@ -65,6 +65,10 @@ inline int num_cus() {
 // 128-row workgroups per compute unit.
 inline bool small_grid(int B, int H, int L) { return (int64_t)B * H * ((L + 127) / 128) < 2 * (int64_t)num_cus(); }
 
+// A short sequence whose last 256-row workgroup would be half empty (an odd number of 128-row
+// blocks, at most three): 128-row workgroups waste nothing there.
+inline bool half_empty_256(int L) { return L <= 384 && ((L + 127) / 128) % 2 == 1; }
+
 // Whether the backward of a call runs the streamlined dk/dv kernel (fb_bwd_dkv_lean.h), which is
 // also whether the writers of the scratch buffer (preprocess step, dq kernel) add the statistics
 // chunks it reads: aligned tensors, no mask, head dim 32 exactly and rank 8 or none (its copies
