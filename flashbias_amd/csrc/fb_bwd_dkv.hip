@@ -438,9 +438,11 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
                     for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[kb][t], s);
                     const bool edge = (wk0 + kb * 32 + 32 > a.Lk) || (a.causal && wk0 + kb * 32 + 31 > m0 + qb * 32);
                     if (edge) {
+                        int query0 = m0 + qb * 32 + 4 * g;
+                        asm volatile("" : "+v"(query0)); // (computed here, not kept in registers across the loop)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int query = m0 + qb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            const int query = query0 + 8 * (v >> 2) + (v & 3);
                             if (key >= a.Lk || (a.causal && key > query)) s[v] = -INFINITY;
                         }
                     }
@@ -497,59 +499,43 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     // ---- epilogue: dv, dk (times scale), dk_bias for this lane's keys
 #pragma unroll
     for (int kb = 0; kb < C::KBW; ++kb) {
-        const int key = wk0 + kb * 32 + c;
-        if (key < a.Lk) {
-            uint16_t *dvrow = const_cast<uint16_t *>(a.dv.ptr) + b * a.dv.sb + h * a.dv.sh + (int64_t)key * a.dv.ss;
-            uint16_t *dkrow = const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + (int64_t)key * a.dk.ss;
-            uint16_t *dkbrow = nullptr;
-            if constexpr (C::NKR > 0)
-                dkbrow = const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + (int64_t)key * a.dkb.ss;
+        int key = wk0 + kb * 32 + c;
+        asm volatile("" : "+v"(key)); // (keeps the address arithmetic below the query loop: its registers are all taken)
+        const bool ok = key < a.Lk;
+        const int64_t krow = ok ? key : 0;
+        uint16_t *dvrow = const_cast<uint16_t *>(a.dv.ptr) + b * a.dv.sb + h * a.dv.sh + krow * a.dv.ss;
+        uint16_t *dkrow = const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + krow * a.dk.ss;
+        uint16_t *dkbrow = nullptr;
+        if constexpr (C::NKR > 0) dkbrow = const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + krow * a.dkb.ss;
 #pragma unroll
-            for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n)
+        for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n)
+            store_acc_rows<T, C::VEC>(dvrow + 32 * n, ok, a.dv.vec_ok, acc_dv[kb][n], 1.f, a.d - 32 * n, g);
+        // block n holds channels [32 n, 32 n + 32) of [dK | dK_b]; dK_b starts at channel 16 NKD (a multiple
+        // of 16, so a 16-channel half of a block is all dk or all dk_bias)
 #pragma unroll
-                for (int bq = 0; bq < 4; ++bq) {
-                    const int ch = 32 * n + 8 * bq + 4 * g;
-                    if (C::VEC && a.dv.vec_ok && ch + 4 <= a.d) {
-                        u32x2_t pk;
-                        pk[0] = T::pack2(acc_dv[kb][n][4 * bq], acc_dv[kb][n][4 * bq + 1]);
-                        pk[1] = T::pack2(acc_dv[kb][n][4 * bq + 2], acc_dv[kb][n][4 * bq + 3]);
-                        *reinterpret_cast<u32x2_t *>(dvrow + ch) = pk;
-                    } else {
+        for (int n = C::MB0; n < C::MB1; ++n) {
+            const f32x16_t &blk = acc_dk[kb][n - C::MB0];
+            if (32 * n + 32 <= 16 * C::NKD) {
+                store_acc_rows<T, C::VEC>(dkrow + 32 * n, ok, a.dk.vec_ok, blk, a.scale, a.d - 32 * n, g);
+            } else if constexpr (C::NKR > 0) {
+                if (32 * n >= 16 * C::NKD) {
+                    const int cr = 32 * n - 16 * C::NKD;
+                    store_acc_rows<T, C::VEC>(dkbrow + cr, ok, a.dkb.vec_ok, blk, 1.f, a.r - cr, g);
+                } else { // the block straddles: channels [32 n, 32 n + 16) are dk, the rest dk_bias
+                    f32x16_t lo, hi;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (ch + e < a.d) dvrow[ch + e] = T::from_float(acc_dv[kb][n][4 * bq + e]);
+                    for (int v = 0; v < 8; ++v) {
+                        lo[v] = blk[v];
+                        lo[8 + v] = 0.f;
+                        hi[v] = blk[8 + v];
+                        hi[8 + v] = 0.f;
                     }
+                    store_acc_rows<T, C::VEC>(dkrow + 32 * n, ok, a.dk.vec_ok, lo, a.scale, min(a.d - 32 * n, 16), g);
+                    store_acc_rows<T, C::VEC>(dkbrow, ok, a.dkb.vec_ok, hi, 1.f, min(a.r, 16), g);
                 }
-#pragma unroll
-            for (int n = C::MB0; n < C::MB1; ++n)
-#pragma unroll
-                for (int bq = 0; bq < 4; ++bq) {
-                    const int ch = 32 * n + 8 * bq + 4 * g;
-                    if (ch < 16 * C::NKD) {
-                        if (C::VEC && a.dk.vec_ok && ch + 4 <= a.d) {
-                            u32x2_t pk;
-                            pk[0] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq] * a.scale, acc_dk[kb][n - C::MB0][4 * bq + 1] * a.scale);
-                            pk[1] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq + 2] * a.scale, acc_dk[kb][n - C::MB0][4 * bq + 3] * a.scale);
-                            *reinterpret_cast<u32x2_t *>(dkrow + ch) = pk;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                if (ch + e < a.d) dkrow[ch + e] = T::from_float(acc_dk[kb][n - C::MB0][4 * bq + e] * a.scale);
-                        }
-                    } else if constexpr (C::NKR > 0) {
-                        const int cr = ch - 16 * C::NKD;
-                        if (C::VEC && a.dkb.vec_ok && cr + 4 <= a.r) {
-                            u32x2_t pk;
-                            pk[0] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq], acc_dk[kb][n - C::MB0][4 * bq + 1]);
-                            pk[1] = T::pack2(acc_dk[kb][n - C::MB0][4 * bq + 2], acc_dk[kb][n - C::MB0][4 * bq + 3]);
-                            *reinterpret_cast<u32x2_t *>(dkbrow + cr) = pk;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                if (cr + e < a.r) dkbrow[cr + e] = T::from_float(acc_dk[kb][n - C::MB0][4 * bq + e]);
-                        }
-                    }
-                }
+            } else {
+                store_acc_rows<T, C::VEC>(dkrow + 32 * n, ok, a.dk.vec_ok, blk, a.scale, a.d - 32 * n, g);
+            }
         }
     }
 }

@@ -401,9 +401,11 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], t == 0 ? negd[qb] : dp);
                     const bool edge = (n0 + kb * 32 + 32 > a.Lk) || (a.causal && n0 + kb * 32 + 31 > wq0 + qb * 32);
                     if (edge) {
+                        int key0 = n0 + kb * 32 + 4 * g;
+                        asm volatile("" : "+v"(key0)); // (computed here, not kept in 16 registers across the loop)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int key = n0 + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            const int key = key0 + 8 * (v >> 2) + (v & 3);
                             if (key >= a.Lk || (a.causal && key > query)) s[v] = -INFINITY;
                         }
                     }
@@ -442,42 +444,38 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     // ---- epilogue: dq = scale * acc rows [0, d), dq_bias = acc rows [16 NKD, 16 NKD + r)
 #pragma unroll
     for (int qb = 0; qb < C::QBLK; ++qb) {
-        const int query = wq0 + qb * 32 + c;
-        if (query < a.Lq) {
-            uint16_t *dqrow = const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + (int64_t)query * a.dq.ss;
-            uint16_t *dqbrow = nullptr;
-            if constexpr (C::NKR > 0)
-                dqbrow = const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + (int64_t)query * a.dqb.ss;
+        int query = wq0 + qb * 32 + c;
+        asm volatile("" : "+v"(query)); // (keeps the address arithmetic below the key loop: its registers are all taken)
+        const bool ok = query < a.Lq;
+        const int64_t qrow = ok ? query : 0;
+        uint16_t *dqrow = const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + qrow * a.dq.ss;
+        uint16_t *dqbrow = nullptr;
+        if constexpr (C::NKR > 0) dqbrow = const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + qrow * a.dqb.ss;
+        // block n holds channels [32 n, 32 n + 32) of [dQ | dQ_b]; dQ_b starts at channel 16 NKD (a multiple
+        // of 16, so a 16-channel half of a block is all dq or all dq_bias)
 #pragma unroll
-            for (int n = 0; n < C::MB; ++n)
+        for (int n = 0; n < C::MB; ++n) {
+            if (32 * n + 32 <= 16 * C::NKD) {
+                store_acc_rows<T, C::VEC>(dqrow + 32 * n, ok, a.dq.vec_ok, acc[qb][n], a.scale, a.d - 32 * n, g);
+            } else if constexpr (C::NKR > 0) {
+                if (32 * n >= 16 * C::NKD) {
+                    const int cr = 32 * n - 16 * C::NKD;
+                    store_acc_rows<T, C::VEC>(dqbrow + cr, ok, a.dqb.vec_ok, acc[qb][n], 1.f, a.r - cr, g);
+                } else { // the block straddles: channels [32 n, 32 n + 16) are dq, the rest dq_bias
+                    f32x16_t lo, hi;
 #pragma unroll
-                for (int bq = 0; bq < 4; ++bq) {
-                    const int ch = 32 * n + 8 * bq + 4 * g; // 4 consecutive channels per lane
-                    if (ch < 16 * C::NKD) {
-                        if (C::VEC && a.dq.vec_ok && ch + 4 <= a.d) {
-                            u32x2_t pk;
-                            pk[0] = T::pack2(acc[qb][n][4 * bq] * a.scale, acc[qb][n][4 * bq + 1] * a.scale);
-                            pk[1] = T::pack2(acc[qb][n][4 * bq + 2] * a.scale, acc[qb][n][4 * bq + 3] * a.scale);
-                            *reinterpret_cast<u32x2_t *>(dqrow + ch) = pk;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                if (ch + e < a.d) dqrow[ch + e] = T::from_float(acc[qb][n][4 * bq + e] * a.scale);
-                        }
-                    } else if constexpr (C::NKR > 0) {
-                        const int cr = ch - 16 * C::NKD;
-                        if (C::VEC && a.dqb.vec_ok && cr + 4 <= a.r) {
-                            u32x2_t pk;
-                            pk[0] = T::pack2(acc[qb][n][4 * bq], acc[qb][n][4 * bq + 1]);
-                            pk[1] = T::pack2(acc[qb][n][4 * bq + 2], acc[qb][n][4 * bq + 3]);
-                            *reinterpret_cast<u32x2_t *>(dqbrow + cr) = pk;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                if (cr + e < a.r) dqbrow[cr + e] = T::from_float(acc[qb][n][4 * bq + e]);
-                        }
+                    for (int v = 0; v < 8; ++v) {
+                        lo[v] = acc[qb][n][v];
+                        lo[8 + v] = 0.f;
+                        hi[v] = acc[qb][n][8 + v];
+                        hi[8 + v] = 0.f;
                     }
+                    store_acc_rows<T, C::VEC>(dqrow + 32 * n, ok, a.dq.vec_ok, lo, a.scale, min(a.d - 32 * n, 16), g);
+                    store_acc_rows<T, C::VEC>(dqbrow, ok, a.dqb.vec_ok, hi, 1.f, min(a.r, 16), g);
                 }
+            } else {
+                store_acc_rows<T, C::VEC>(dqrow + 32 * n, ok, a.dq.vec_ok, acc[qb][n], a.scale, a.d - 32 * n, g);
+            }
         }
     }
 }

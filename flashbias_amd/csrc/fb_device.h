@@ -433,6 +433,40 @@ __device__ __forceinline__ float half_wave_max(float x) {
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Epilogue store of one 32 x 32 accumulator block whose lanes are rows: lane (c, g) holds, for
+// bq = 0..3, the channels ch0 + 8 bq + 4 g + {0..3} of row c in acc[4 bq .. 4 bq + 3] (what the
+// 32x32 MFMA leaves with the row operand as B).  `row` points at channel ch0 of this lane's row,
+// `ncols` counts the channels from ch0 that exist, `mul` scales the values.  With 16-byte aligned
+// rows (`vec`, ncols a multiple of 8) the two lanes of a row first exchange halves
+// (v_permlane32_swap: the upper half of one register against the lower half of another), so that
+// each stores 16 contiguous bytes and the pair a 32-byte piece of the row: half the store
+// instructions and write requests of 8-byte stores.  Must be called by all lanes (the exchange is
+// outside the row test).
+template <class T, bool VEC>
+__device__ __forceinline__ void store_acc_rows(uint16_t *row, bool row_ok, bool vec, const f32x16_t &acc, float mul,
+                                               int ncols, int g) {
+    if (VEC && vec) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            uint32_t e0 = T::pack2(acc[8 * j] * mul, acc[8 * j + 1] * mul), e1 = T::pack2(acc[8 * j + 2] * mul, acc[8 * j + 3] * mul);
+            uint32_t o0 = T::pack2(acc[8 * j + 4] * mul, acc[8 * j + 5] * mul), o1 = T::pack2(acc[8 * j + 6] * mul, acc[8 * j + 7] * mul);
+            // lower half-wave: (e, o) = channels 16 j + {0..3, 4..7}; upper: channels 16 j + {8..11, 12..15}
+            asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+                         : "+v"(e0), "+v"(o0), "+v"(e1), "+v"(o1));
+            const int col = 16 * j + 8 * g;
+            if (row_ok && col + 8 <= ncols) *reinterpret_cast<u32x4_t *>(row + col) = u32x4_t{e0, e1, o0, o1};
+        }
+    } else if (row_ok) {
+#pragma unroll
+        for (int bq = 0; bq < 4; ++bq)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int col = 8 * bq + 4 * g + e;
+                if (col < ncols) row[col] = T::from_float(acc[4 * bq + e] * mul);
+            }
+    }
+}
+
 // Turn-taking between the workgroups that share a CU.  The instruction arbiter serves the oldest
 // wave of a SIMD first, so of two resident workgroups the older one runs at the speed it would
 // have alone and the younger one only fills its stalls: their progress differs by a third, and

@@ -443,11 +443,13 @@ __device__ __forceinline__ void fwd_body(const FwdArgs &a) {
                 const bool ragged = ns + C::BSUB > a.Lk;
                 const bool diag = a.causal && (ns + C::BSUB - 1 > bq0);
                 if (ragged || diag) {
+                    int key0 = ns + 4 * g;
+                    asm volatile("" : "+v"(key0)); // (computed here, not kept in registers across the loop)
 #pragma unroll
                     for (int kb = 0; kb < C::KBLK; ++kb)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) {
-                            const int key = ns + kb * 32 + 8 * (v >> 2) + 4 * g + (v & 3);
+                            const int key = key0 + kb * 32 + 8 * (v >> 2) + (v & 3);
                             if (key >= a.Lk || (a.causal && key > query)) s[kb][v] = -INFINITY;
                         }
                 }
@@ -505,29 +507,15 @@ __device__ __forceinline__ void fwd_body(const FwdArgs &a) {
     uint16_t *obase = const_cast<uint16_t *>(a.o.ptr) + b * a.o.sb + h * a.o.sh;
 #pragma unroll
     for (int qb = 0; qb < C::QB; ++qb) {
-        const int query = wq0 + 32 * qb + c;
+        int query = wq0 + 32 * qb + c;
+        asm volatile("" : "+v"(query)); // (keeps the address arithmetic below the key loop)
         const float l = l_run[qb] + __shfl_xor(l_run[qb], 32, 64);
         const float inv = 1.f / l;
-        if (query < a.Lq) {
-            if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref[qb] * (C::FOLD ? a.scale : 1.f) + __builtin_amdgcn_logf(l) * kLn2;
-            uint16_t *orow = obase + (int64_t)query * a.o.ss;
+        const bool ok = query < a.Lq;
+        if (ok && g == 0) a.lse[(int64_t)bh * a.Lq + query] = m_ref[qb] * (C::FOLD ? a.scale : 1.f) + __builtin_amdgcn_logf(l) * kLn2;
+        uint16_t *orow = obase + (int64_t)(ok ? query : 0) * a.o.ss;
 #pragma unroll
-            for (int n = 0; n < C::NDV; ++n)
-#pragma unroll
-                for (int bq = 0; bq < 4; ++bq) {
-                    const int ch = 32 * n + 8 * bq + 4 * g;
-                    if (C::VEC && ch + 4 <= a.d) {
-                        u32x2_t pk;
-                        pk[0] = T::pack2(acc_o[qb][n][4 * bq] * inv, acc_o[qb][n][4 * bq + 1] * inv);
-                        pk[1] = T::pack2(acc_o[qb][n][4 * bq + 2] * inv, acc_o[qb][n][4 * bq + 3] * inv);
-                        *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (ch + e < a.d) orow[ch + e] = T::from_float(acc_o[qb][n][4 * bq + e] * inv);
-                    }
-                }
-        }
+        for (int n = 0; n < C::NDV; ++n) store_acc_rows<T, C::VEC>(orow + 32 * n, ok, true, acc_o[qb][n], inv, a.d - 32 * n, g);
     }
 }
 
