@@ -344,43 +344,15 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dv), "+v"(acc_dk), "+v"(acc_dkb));
     else
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dv), "+v"(acc_dk));
-    if (key < a.Lk) {
-        uint16_t *dvrow = const_cast<uint16_t *>(a.dv.ptr) + b * a.dv.sb + h * a.dv.sh + (int64_t)key * a.dv.ss;
-        uint16_t *dkrow = const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + (int64_t)key * a.dk.ss;
-#pragma unroll
-        for (int bq = 0; bq < 4; ++bq) {
-            const int ch = 8 * bq + 4 * g;
-            u32x2_t pv, pk;
-            pv[0] = T::pack2(acc_dv[4 * bq], acc_dv[4 * bq + 1]);
-            pv[1] = T::pack2(acc_dv[4 * bq + 2], acc_dv[4 * bq + 3]);
-            pk[0] = T::pack2(acc_dk[4 * bq] * a.scale, acc_dk[4 * bq + 1] * a.scale);
-            pk[1] = T::pack2(acc_dk[4 * bq + 2] * a.scale, acc_dk[4 * bq + 3] * a.scale);
-            if (a.dv.vec_ok)
-                *reinterpret_cast<u32x2_t *>(dvrow + ch) = pv;
-            else {
-                dvrow[ch] = (uint16_t)pv[0]; dvrow[ch + 1] = (uint16_t)(pv[0] >> 16);
-                dvrow[ch + 2] = (uint16_t)pv[1]; dvrow[ch + 3] = (uint16_t)(pv[1] >> 16);
-            }
-            if (a.dk.vec_ok)
-                *reinterpret_cast<u32x2_t *>(dkrow + ch) = pk;
-            else {
-                dkrow[ch] = (uint16_t)pk[0]; dkrow[ch + 1] = (uint16_t)(pk[0] >> 16);
-                dkrow[ch + 2] = (uint16_t)pk[1]; dkrow[ch + 3] = (uint16_t)(pk[1] >> 16);
-            }
-        }
-        if constexpr (NKR > 0) { // rows 0..7 of the third accumulator block (8..15 repeat them)
-            uint16_t *dkbrow = const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + (int64_t)key * a.dkb.ss;
-            u32x2_t pb;
-            pb[0] = T::pack2(acc_dkb[0], acc_dkb[1]);
-            pb[1] = T::pack2(acc_dkb[2], acc_dkb[3]);
-            if (a.dkb.vec_ok)
-                *reinterpret_cast<u32x2_t *>(dkbrow + 4 * g) = pb;
-            else {
-                dkbrow[4 * g] = (uint16_t)pb[0]; dkbrow[4 * g + 1] = (uint16_t)(pb[0] >> 16);
-                dkbrow[4 * g + 2] = (uint16_t)pb[1]; dkbrow[4 * g + 3] = (uint16_t)(pb[1] >> 16);
-            }
-        }
-    }
+    const bool ok = key < a.Lk;
+    const int64_t krow = ok ? key : 0;
+    store_acc_rows<T, true>(const_cast<uint16_t *>(a.dv.ptr) + b * a.dv.sb + h * a.dv.sh + krow * a.dv.ss, ok, a.dv.vec_ok, acc_dv, 1.f,
+                            32, g);
+    store_acc_rows<T, true>(const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + krow * a.dk.ss, ok, a.dk.vec_ok, acc_dk,
+                            a.scale, 32, g);
+    if constexpr (NKR > 0) // rows 0..7 of the third accumulator block (8..15 repeat them)
+        store_acc_rows<T, true>(const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + krow * a.dkb.ss, ok, a.dkb.vec_ok,
+                                acc_dkb, 1.f, 8, g);
 }
 
 template <class T, int NKR>

@@ -352,34 +352,12 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dq), "+v"(acc_dqb));
     else
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dq));
-    if (ok) {
-        uint16_t *dqrow = const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + (int64_t)query * a.dq.ss;
-#pragma unroll
-        for (int bq = 0; bq < 4; ++bq) {
-            const int ch = 8 * bq + 4 * g;
-            u32x2_t pk;
-            pk[0] = T::pack2(acc_dq[4 * bq] * a.scale, acc_dq[4 * bq + 1] * a.scale);
-            pk[1] = T::pack2(acc_dq[4 * bq + 2] * a.scale, acc_dq[4 * bq + 3] * a.scale);
-            if (a.dq.vec_ok)
-                *reinterpret_cast<u32x2_t *>(dqrow + ch) = pk;
-            else {
-                dqrow[ch] = (uint16_t)pk[0]; dqrow[ch + 1] = (uint16_t)(pk[0] >> 16);
-                dqrow[ch + 2] = (uint16_t)pk[1]; dqrow[ch + 3] = (uint16_t)(pk[1] >> 16);
-            }
-        }
-        if constexpr (NKR > 0) { // rows 0..7 of the second accumulator block (8..15 repeat them)
-            uint16_t *dqbrow = const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + (int64_t)query * a.dqb.ss;
-            u32x2_t pb;
-            pb[0] = T::pack2(acc_dqb[0], acc_dqb[1]);
-            pb[1] = T::pack2(acc_dqb[2], acc_dqb[3]);
-            if (a.dqb.vec_ok)
-                *reinterpret_cast<u32x2_t *>(dqbrow + 4 * g) = pb;
-            else {
-                dqbrow[4 * g] = (uint16_t)pb[0]; dqbrow[4 * g + 1] = (uint16_t)(pb[0] >> 16);
-                dqbrow[4 * g + 2] = (uint16_t)pb[1]; dqbrow[4 * g + 3] = (uint16_t)(pb[1] >> 16);
-            }
-        }
-    }
+    const int64_t qrow = ok ? query : 0;
+    store_acc_rows<T, true>(const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + qrow * a.dq.ss, ok, a.dq.vec_ok, acc_dq,
+                            a.scale, 32, g);
+    if constexpr (NKR > 0) // rows 0..7 of the second accumulator block (8..15 repeat them)
+        store_acc_rows<T, true>(const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + qrow * a.dqb.ss, ok, a.dqb.vec_ok,
+                                acc_dqb, 1.f, 8, g);
 }
 
 template <class T, int NKR>

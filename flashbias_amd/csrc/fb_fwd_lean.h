@@ -345,18 +345,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         const int query = wq0 + 32 * qb + c;
         const float l = l_run[qb];
         const float inv = 1.f / l;
-        if (query < a.Lq) {
-            if (g == 0) a.lse[(int64_t)bh * a.Lq + query] = (m2 + __builtin_amdgcn_logf(l)) * kLn2;
-            uint16_t *orow = obase + (int64_t)query * a.o.ss;
-#pragma unroll
-            for (int bq = 0; bq < 4; ++bq) {
-                const int ch = 8 * bq + 4 * g;
-                u32x2_t pk;
-                pk[0] = T::pack2(acc_o[qb][4 * bq] * inv, acc_o[qb][4 * bq + 1] * inv);
-                pk[1] = T::pack2(acc_o[qb][4 * bq + 2] * inv, acc_o[qb][4 * bq + 3] * inv);
-                *reinterpret_cast<u32x2_t *>(orow + ch) = pk;
-            }
-        }
+        const bool ok = query < a.Lq;
+        if (ok && g == 0) a.lse[(int64_t)bh * a.Lq + query] = (m2 + __builtin_amdgcn_logf(l)) * kLn2;
+        store_acc_rows<T, true>(obase + (int64_t)(ok ? query : 0) * a.o.ss, ok, true, acc_o[qb], inv, 32, g);
     }
 }
 
