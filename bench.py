@@ -165,6 +165,44 @@ def _autograd_ms(leaves, extra, do, steps, warmup, prepare=None):
     return t_fwd, _time_events(fb, steps, warmup)
 
 
+def _graph_ms(leaves, extra, do, steps, warmup):
+    """fwd+bwd milliseconds of the same autograd step captured once in a HIP graph and replayed: what
+    a training loop that captures its step pays, without the host's per-call work (which bounds the
+    eager figure when the kernels of a step take less than about 0.1 ms).  Every replay's gradients
+    are compared with the eager step's bit for bit; returns None if they differ or capture fails."""
+    import torch
+    from flashbias_amd import flash_bias_func
+    mask, causal, scale = extra
+
+    def step():
+        o = flash_bias_func(leaves[0], leaves[1], leaves[2], leaves[3], leaves[4], mask, causal, scale)
+        return torch.autograd.grad(o, leaves, do)
+
+    eager = [g.clone() for g in step()]
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            grads = step()
+        for _ in range(max(1, warmup)):
+            graph.replay()
+            torch.cuda.synchronize()
+            if not all(torch.equal(a, b) for a, b in zip(grads, eager)):
+                return None
+        ms = _time_events(graph.replay, steps, 0)
+        torch.cuda.synchronize()
+        if not all(torch.equal(a, b) for a, b in zip(grads, eager)):
+            return None
+        return ms
+    except RuntimeError:
+        return None
+
+
 def _device_configs(dev):
     """(name, builder) of every benchmark configuration at its stated size; q, k, v, dO are drawn on
     the device (timing does not depend on the values), the factors come from the builders."""
@@ -219,6 +257,7 @@ def _sweep(dev, steps, warmup, only=None):
         B, L, H, d = q.shape
         leaves = [t.requires_grad_(True) for t in (q, k, v, qb, kb)]
         t_fwd, t_fb = _autograd_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
+        t_graph = _graph_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
         f_fwd, f_bwd = workloads.flops(B, H, L, L, d, r, causal)
         # algorithmic HBM bytes of a step: every input read once per pass, every output written once
         # (forward: q k v factors -> o, lse; backward: q k v o dO factors lse -> dq dk dv and the factor
@@ -229,6 +268,9 @@ def _sweep(dev, steps, warmup, only=None):
         out.append({"workload": name, "fwd_ms": round(t_fwd, 4), "fwd_bwd_ms": round(t_fb, 4),
                     "fwd_tflops": round(f_fwd / t_fwd / 1e9, 1), "fwd_bwd_tflops": round((f_fwd + f_bwd) / t_fb / 1e9, 1),
                     "pct_of_bf16_mfma_peak": round(100 * (f_fwd + f_bwd) / t_fb / 1e9 / PEAK_BF16_TFLOPS, 2),
+                    "fwd_bwd_graph_ms": None if t_graph is None else round(t_graph, 4),
+                    "graph_pct_of_bf16_mfma_peak": None if t_graph is None else
+                    round(100 * (f_fwd + f_bwd) / t_graph / 1e9 / PEAK_BF16_TFLOPS, 2),
                     "hbm_algorithmic_gb": round(hbm / 1e9, 3), "hbm_gbs": round(hbm / t_fb / 1e6, 1),
                     "pct_of_hbm_peak": round(100 * hbm / t_fb / 1e6 / PEAK_HBM_GBS, 2)})
         del q, k, v, qb, kb, do, leaves
