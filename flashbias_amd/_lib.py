@@ -13,7 +13,8 @@ FB_F16, FB_BF16, FB_F32 = 0, 1, 2
 FB_MASK_NONE, FB_MASK_VECTOR, FB_MASK_MATRIX = 0, 1, 2
 
 #: every symbol that include/flashbias.h declares
-EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_check", "fb_fwd", "fb_bwd", "fb_sum_over_batch",
+EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_suggest_bias_grad_group", "fb_check", "fb_fwd", "fb_bwd",
+           "fb_sum_over_batch",
            "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static")
 
 
@@ -30,7 +31,7 @@ class FbParams(ctypes.Structure):
                 + [(n, FbTensor) for n in ("q", "k", "v", "q_bias", "k_bias", "mask", "o")]
                 + [("lse", ctypes.c_void_p)]
                 + [(n, FbTensor) for n in ("dout", "dq", "dk", "dv", "dq_bias", "dk_bias")]
-                + [("delta", ctypes.c_void_p)])
+                + [("delta", ctypes.c_void_p), ("bias_grad_group", ctypes.c_int32)])
 
 
 class FlashBiasError(RuntimeError):
@@ -61,6 +62,8 @@ def load():
     lib.fb_last_error.restype = ctypes.c_char_p
     lib.fb_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FbParams)]
     lib.fb_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.fb_suggest_bias_grad_group.argtypes = [ctypes.POINTER(FbParams)]
+    lib.fb_suggest_bias_grad_group.restype = ctypes.c_int
     lib.fb_check.argtypes = [ctypes.POINTER(FbParams), ctypes.c_int]
     lib.fb_check.restype = ctypes.c_int
     for name in ("fb_fwd", "fb_bwd", "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static"):

@@ -151,6 +151,7 @@ fb::BwdArgs bwd_args(const fb_params *p) {
     a.B = p->B; a.H = p->H; a.Lq = p->Lq; a.Lk = p->Lk; a.d = p->d; a.r = p->r;
     a.causal = p->causal ? 1 : 0;
     a.scale = p->scale;
+    a.group = p->r > 0 && p->bias_grad_group > 1 ? p->bias_grad_group : 1;
     a.stat_chunks = fb::dkv_streamlined(a) ? 1 : 0;
     return a;
 }

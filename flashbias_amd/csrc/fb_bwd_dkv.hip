@@ -229,6 +229,55 @@ struct DkvDirect {
     }
 };
 
+// Epilogue stores of the dk/dv kernel: dv and the dk part of the accumulators (BIAS = false, batch
+// row `brow`) or their dk_bias part (BIAS = true, batch row `brow` of dk_bias).  Block n of acc_dk
+// holds channels [32 n, 32 n + 32) of [dK | dK_b]; dK_b starts at channel 16 NKD (a multiple of 16,
+// so a 16-channel half of a block is all dk or all dk_bias).
+template <class T, class C, bool BIAS>
+__device__ __forceinline__ void dkv_store(const BwdArgs &a, const f32x16_t (&acc_dv)[C::KBW][C::DO_DV ? C::NDV : 1],
+                                          const f32x16_t (&acc_dk)[C::KBW][C::DO_DK ? C::MB1 - C::MB0 : 1], int brow, int h,
+                                          int wk0, int c, int g) {
+    const Tensor &t = BIAS ? a.dkb : a.dk;
+    const float mul = BIAS ? 1.f : a.scale;
+    const int ncols = BIAS ? a.r : a.d;
+    constexpr int CH0 = BIAS ? 16 * C::NKD : 0;          // first channel of this part in [dK | dK_b]
+    constexpr int END = BIAS ? 32 * C::MB : 16 * C::NKD; // one past its last channel
+#pragma unroll
+    for (int kb = 0; kb < C::KBW; ++kb) {
+        int key = wk0 + kb * 32 + c;
+        asm volatile("" : "+v"(key)); // (keeps the address arithmetic below the query loop: its registers are all taken)
+        const bool ok = key < a.Lk;
+        const int64_t krow = ok ? key : 0;
+        if constexpr (!BIAS && C::DO_DV) {
+            uint16_t *dvrow = const_cast<uint16_t *>(a.dv.ptr) + brow * a.dv.sb + h * a.dv.sh + krow * a.dv.ss;
+#pragma unroll
+            for (int n = 0; n < C::NDV; ++n)
+                store_acc_rows<T, C::VEC>(dvrow + 32 * n, ok, a.dv.vec_ok, acc_dv[kb][n], 1.f, a.d - 32 * n, g);
+        }
+        if constexpr (C::DO_DK) {
+            uint16_t *row = const_cast<uint16_t *>(t.ptr) + brow * t.sb + h * t.sh + krow * t.ss;
+#pragma unroll
+            for (int n = C::MB0; n < C::MB1; ++n) {
+                const f32x16_t &blk = acc_dk[kb][n - C::MB0];
+                const int lo_ch = 32 * n, hi_ch = 32 * n + 32;
+                if (hi_ch <= CH0 || lo_ch >= END) continue; // the block has nothing of this part
+                if (lo_ch >= CH0 && hi_ch <= END) {
+                    store_acc_rows<T, C::VEC>(row + (lo_ch - CH0), ok, t.vec_ok, blk, mul, ncols - (lo_ch - CH0), g);
+                } else { // the block straddles: channels [32 n, 32 n + 16) are dk, the rest dk_bias
+                    f32x16_t half;
+#pragma unroll
+                    for (int v = 0; v < 8; ++v) {
+                        half[v] = blk[BIAS ? 8 + v : v];
+                        half[8 + v] = 0.f;
+                    }
+                    const int off = BIAS ? 0 : lo_ch;
+                    store_acc_rows<T, C::VEC>(row + off, ok, t.vec_ok, half, mul, min(ncols - off, 16), g);
+                }
+            }
+        }
+    }
+}
+
 template <class T, class C>
 __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -238,13 +287,45 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 31, g = lane >> 5;
 
-    const int total = a.ntiles_n * a.B * a.H;
+    // One workgroup serves `group` consecutive batch entries of its (head, key tile), one after the
+    // other: dk and dv are written per entry, the dk_bias accumulators run on and are written once, as
+    // row b / group of the dk_bias tensor (factors shared by the batch: their gradient is the sum).
+    const int group = a.group > 1 ? a.group : 1;
+    const int nbg = (a.B + group - 1) / group;
+    const int total = a.ntiles_n * nbg * a.H;
     const int work = xcd_remap(blockIdx.x, total);
-    const int bh = work / a.ntiles_n;
+    const int bgh = work / a.ntiles_n;
     const int tile_n = work % a.ntiles_n; // causal: low key tiles see the most queries, they go first
-    const int b = bh / a.H, h = bh % a.H;
+    const int bg = bgh / a.H, h = bgh % a.H;
     const int n0 = tile_n * C::BN;
     const int wk0 = n0 + wave * (32 * C::KBW); // first key of this wave
+
+    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
+        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
+        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+
+    f32x16_t acc_dv[C::KBW][C::DO_DV ? C::NDV : 1], acc_dk[C::KBW][C::DO_DK ? C::MB1 - C::MB0 : 1];
+#pragma unroll
+    for (int kb = 0; kb < C::KBW; ++kb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+#pragma unroll
+            for (int n = 0; n < (C::DO_DV ? C::NDV : 1); ++n) acc_dv[kb][n][v] = 0.f;
+#pragma unroll
+            for (int n = 0; n < (C::DO_DK ? C::MB1 - C::MB0 : 1); ++n) acc_dk[kb][n][v] = 0.f;
+        }
+
+    for (int bi = 0; bi < group; ++bi) {
+    const int b = __builtin_amdgcn_readfirstlane(bg * group + bi); // (wave-uniform, and the compiler should know)
+    if (b >= a.B) break;
+    // (the lane's coordinates again, opaque to the compiler: what it derives from them is computed per batch
+    // entry, as in a workgroup of its own, instead of being kept in registers across this loop)
+    int tid_again = threadIdx.x;
+    asm volatile("" : "+v"(tid_again));
+    const int tid = tid_again, lane = tid & 63, c = lane & 31, g = lane >> 5;
+    const int bh = b * a.H + h;
 
     const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
     const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
@@ -268,7 +349,6 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     // ---- key-side operands, resident in registers
     u32x4_t kreg[C::KBW][C::NK];  // B operand of S: this lane's key, channels 16t + 8g ..
     u32x4_t vreg[C::KBW][C::DO_DK ? C::NKD : 1]; // B operand of dP
-    f32x16_t acc_dv[C::KBW][C::DO_DV ? C::NDV : 1], acc_dk[C::KBW][C::DO_DK ? C::MB1 - C::MB0 : 1];
 #pragma unroll
     for (int kb = 0; kb < C::KBW; ++kb) {
         const int key = wk0 + kb * 32 + c;
@@ -287,12 +367,14 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
             for (int t = 0; t < C::NKD; ++t)
                 vreg[kb][t] = load_chunk<C::VEC>(vbase, a.v.ss, key, a.Lk, 16 * t + 8 * g, a.d);
         }
+        // (element v of block n is channel 32 n + 8 (v / 4) + 4 g + v % 4: below 16 NKD it belongs to dk)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
 #pragma unroll
             for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n) acc_dv[kb][n][v] = 0.f;
 #pragma unroll
-            for (int n = 0; n < C::MB1 - C::MB0; ++n) acc_dk[kb][n][v] = 0.f;
+            for (int n = C::MB0; n < C::MB1; ++n)
+                if (32 * n + 8 * (v >> 2) < 16 * C::NKD) acc_dk[kb][n - C::MB0][v] = 0.f;
         }
     }
 
@@ -300,11 +382,6 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     const int step0 = a.causal ? n0 / C::BMQ : 0;
     const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
 
-    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
-        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
-        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
-    }
-    __syncthreads();
     // Step s is computed from stage (s - step0) % NSTAGE.  Direct loader: the tiles of step
     // s + AHEAD are requested at the top of step s; element-wise loader: step s + 1 goes through
     // registers.
@@ -496,47 +573,14 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
         }
     }
 
-    // ---- epilogue: dv, dk (times scale), dk_bias for this lane's keys
-#pragma unroll
-    for (int kb = 0; kb < C::KBW; ++kb) {
-        int key = wk0 + kb * 32 + c;
-        asm volatile("" : "+v"(key)); // (keeps the address arithmetic below the query loop: its registers are all taken)
-        const bool ok = key < a.Lk;
-        const int64_t krow = ok ? key : 0;
-        uint16_t *dvrow = const_cast<uint16_t *>(a.dv.ptr) + b * a.dv.sb + h * a.dv.sh + krow * a.dv.ss;
-        uint16_t *dkrow = const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + krow * a.dk.ss;
-        uint16_t *dkbrow = nullptr;
-        if constexpr (C::NKR > 0) dkbrow = const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + krow * a.dkb.ss;
-#pragma unroll
-        for (int n = 0; n < (C::DO_DV ? C::NDV : 0); ++n)
-            store_acc_rows<T, C::VEC>(dvrow + 32 * n, ok, a.dv.vec_ok, acc_dv[kb][n], 1.f, a.d - 32 * n, g);
-        // block n holds channels [32 n, 32 n + 32) of [dK | dK_b]; dK_b starts at channel 16 NKD (a multiple
-        // of 16, so a 16-channel half of a block is all dk or all dk_bias)
-#pragma unroll
-        for (int n = C::MB0; n < C::MB1; ++n) {
-            const f32x16_t &blk = acc_dk[kb][n - C::MB0];
-            if (32 * n + 32 <= 16 * C::NKD) {
-                store_acc_rows<T, C::VEC>(dkrow + 32 * n, ok, a.dk.vec_ok, blk, a.scale, a.d - 32 * n, g);
-            } else if constexpr (C::NKR > 0) {
-                if (32 * n >= 16 * C::NKD) {
-                    const int cr = 32 * n - 16 * C::NKD;
-                    store_acc_rows<T, C::VEC>(dkbrow + cr, ok, a.dkb.vec_ok, blk, 1.f, a.r - cr, g);
-                } else { // the block straddles: channels [32 n, 32 n + 16) are dk, the rest dk_bias
-                    f32x16_t lo, hi;
-#pragma unroll
-                    for (int v = 0; v < 8; ++v) {
-                        lo[v] = blk[v];
-                        lo[8 + v] = 0.f;
-                        hi[v] = blk[8 + v];
-                        hi[8 + v] = 0.f;
-                    }
-                    store_acc_rows<T, C::VEC>(dkrow + 32 * n, ok, a.dk.vec_ok, lo, a.scale, min(a.d - 32 * n, 16), g);
-                    store_acc_rows<T, C::VEC>(dkbrow, ok, a.dkb.vec_ok, hi, 1.f, min(a.r, 16), g);
-                }
-            } else {
-                store_acc_rows<T, C::VEC>(dkrow + 32 * n, ok, a.dk.vec_ok, blk, a.scale, a.d - 32 * n, g);
-            }
-        }
+    // ---- epilogue of this batch entry: dv and dk (times scale) for this lane's keys
+    dkv_store<T, C, false>(a, acc_dv, acc_dk, b, h, wk0, c, g);
+    } // batch entries of the group
+
+    // ---- dk_bias, summed over the group's batch entries
+    if constexpr (C::NKR > 0 && C::DO_DK) {
+        const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        dkv_store<T, C, true>(a, acc_dv, acc_dk, bg, h, wk0, lane_end & 31, lane_end >> 5);
     }
 }
 
@@ -555,7 +599,8 @@ static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
     static KernelOnce once;
     const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
     if (e != hipSuccess) return e;
-    return launch_flat(kern, (int64_t)a.ntiles_n * a.B * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
+    const int group = a.group > 1 ? a.group : 1;
+    return launch_flat(kern, (int64_t)a.ntiles_n * ((a.B + group - 1) / group) * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
 }
 
 // One pass, or (head dims above 64, aligned tensors) two or three passes that each keep a part

@@ -164,6 +164,44 @@ struct DqDirect {
     int m0_ = 0; // first query of the workgroup (set by init_mask)
 };
 
+// Epilogue stores of the dq kernel: the dq part (BIAS = false, times the softmax scale, batch row
+// `brow` of dq) or the dq_bias part (BIAS = true, batch row `brow` of dq_bias) of the accumulators.
+// Block n holds channels [32 n, 32 n + 32) of [dQ | dQ_b]; dQ_b starts at channel 16 NKD (a multiple
+// of 16, so a 16-channel half of a block is all dq or all dq_bias).
+template <class T, class C, bool BIAS>
+__device__ __forceinline__ void dq_store(const BwdArgs &a, const f32x16_t (&acc)[C::QBLK][C::MB], int brow, int h, int wq0,
+                                         int c, int g) {
+    const Tensor &t = BIAS ? a.dqb : a.dq;
+    const float mul = BIAS ? 1.f : a.scale;
+    const int ncols = BIAS ? a.r : a.d;
+    constexpr int CH0 = BIAS ? 16 * C::NKD : 0; // first channel of this part in [dQ | dQ_b]
+#pragma unroll
+    for (int qb = 0; qb < C::QBLK; ++qb) {
+        int query = wq0 + qb * 32 + c;
+        asm volatile("" : "+v"(query)); // (keeps the address arithmetic below the key loop: its registers are all taken)
+        const bool ok = query < a.Lq;
+        uint16_t *row = const_cast<uint16_t *>(t.ptr) + brow * t.sb + h * t.sh + (int64_t)(ok ? query : 0) * t.ss;
+#pragma unroll
+        for (int n = 0; n < C::MB; ++n) {
+            constexpr int END = BIAS ? 32 * C::MB : 16 * C::NKD; // one past the last channel of this part
+            const int lo_ch = 32 * n, hi_ch = 32 * n + 32;
+            if (hi_ch <= CH0 || lo_ch >= END) continue; // the block has nothing of this part
+            if (lo_ch >= CH0 && hi_ch <= END) {
+                store_acc_rows<T, C::VEC>(row + (lo_ch - CH0), ok, t.vec_ok, acc[qb][n], mul, ncols - (lo_ch - CH0), g);
+            } else { // the block straddles: channels [32 n, 32 n + 16) are dq, the rest dq_bias
+                f32x16_t half;
+#pragma unroll
+                for (int v = 0; v < 8; ++v) {
+                    half[v] = acc[qb][n][BIAS ? 8 + v : v];
+                    half[8 + v] = 0.f;
+                }
+                const int off = BIAS ? 0 : lo_ch;
+                store_acc_rows<T, C::VEC>(row + off, ok, t.vec_ok, half, mul, min(ncols - off, 16), g);
+            }
+        }
+    }
+}
+
 // The whole dq / dq_bias computation of one workgroup; the kernel below is nothing else.
 template <class T, class C>
 __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
@@ -174,14 +212,44 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int c = lane & 31, g = lane >> 5;
 
-    const int total = a.ntiles_m * a.B * a.H;
+    // One workgroup serves `group` consecutive batch entries of its (head, query tile), one after the
+    // other: dq is written per entry, the dq_bias accumulators run on and are written once, as row
+    // b / group of the dq_bias tensor (factors shared by the batch: their gradient is the sum).
+    const int group = a.group > 1 ? a.group : 1;
+    const int nbg = (a.B + group - 1) / group;
+    const int total = a.ntiles_m * nbg * a.H;
     const int work = xcd_remap(blockIdx.x, total);
-    const int bh = work / a.ntiles_m;
+    const int bgh = work / a.ntiles_m;
     int tile_m = work % a.ntiles_m;
     if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
-    const int b = bh / a.H, h = bh % a.H;
+    const int bg = bgh / a.H, h = bgh % a.H;
     const int m0 = tile_m * C::BM;
     const int wq0 = m0 + wave * (32 * C::QBLK);
+
+    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
+        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
+        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+
+    f32x16_t acc[C::QBLK][C::MB];
+#pragma unroll
+    for (int qb = 0; qb < C::QBLK; ++qb)
+#pragma unroll
+        for (int n = 0; n < C::MB; ++n)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[qb][n][v] = 0.f;
+    int turn = __builtin_amdgcn_readfirstlane(cu_slot());
+
+    for (int bi = 0; bi < group; ++bi) {
+    const int b = __builtin_amdgcn_readfirstlane(bg * group + bi); // (wave-uniform, and the compiler should know)
+    if (b >= a.B) break;
+    // (the lane's coordinates again, opaque to the compiler: what it derives from them is computed per batch
+    // entry, as in a workgroup of its own, instead of being kept in registers across this loop)
+    int tid_again = threadIdx.x;
+    asm volatile("" : "+v"(tid_again));
+    const int tid = tid_again, lane = tid & 63, c = lane & 31, g = lane >> 5;
+    const int bh = b * a.H + h;
 
     const uint16_t *qbase = a.q.ptr + b * a.q.sb + h * a.q.sh;
     const uint16_t *kbase = a.k.ptr + b * a.k.sb + h * a.k.sh;
@@ -204,7 +272,6 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     // -delta of this lane's query in all 16 registers of an accumulator block: the initial value
     // of every dP^T chain (lane = query, so it is the same for every key), no add per score
     f32x16_t negd[C::QBLK];
-    f32x16_t acc[C::QBLK][C::MB];
 #pragma unroll
     for (int qb = 0; qb < C::QBLK; ++qb) {
         const int query = wq0 + qb * 32 + c;
@@ -266,10 +333,12 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
         lse2[qb] = l2; // rows past the end: P = exp2(-inf) = 0
 #pragma unroll
         for (int v = 0; v < 16; ++v) negd[qb][v] = nd;
+        // (element v of block n is channel 32 n + 8 (v / 4) + 4 g + v % 4: below 16 NKD it belongs to dq)
 #pragma unroll
         for (int n = 0; n < C::MB; ++n)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[qb][n][v] = 0.f;
+            for (int v = 0; v < 16; ++v)
+                if (32 * n + 8 * (v >> 2) < 16 * C::NKD) acc[qb][n][v] = 0.f;
     }
 
     const float to_log2 = C::FOLD ? a.scale * kLog2e : kLog2e; // the scores are in units of 1 / scale when folded
@@ -278,11 +347,6 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     if (a.causal && m0 + C::BM < k_end) k_end = m0 + C::BM; // keys past the last query are hidden
     const int ntiles_k = (k_end + C::BN - 1) / C::BN;
 
-    {   // clear the stages once: the zero padding of the channel dimension is never rewritten
-        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
-        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
-    }
-    __syncthreads();
     // Tile t is computed from stage t % NSTAGE.  Direct loader: tile t + 2 is requested at the top
     // of tile t; element-wise loader: tile t + 1 goes through registers.  Keys past the end of a
     // ragged last tile hold copies of the last key; their scores are set to -inf below.
@@ -311,7 +375,6 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     __syncthreads();
 
     int cur = 0; // stage of the current tile
-    int turn = __builtin_amdgcn_readfirstlane(cu_slot());
     take_turn(turn, a.slots);
     for (int it = 0; it < ntiles_k; ++it) {
         const int n0 = it * C::BN;
@@ -441,42 +504,14 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
         take_turn(turn, a.slots); // (next to the barrier: the compiler moves nothing across either)
     }
 
-    // ---- epilogue: dq = scale * acc rows [0, d), dq_bias = acc rows [16 NKD, 16 NKD + r)
-#pragma unroll
-    for (int qb = 0; qb < C::QBLK; ++qb) {
-        int query = wq0 + qb * 32 + c;
-        asm volatile("" : "+v"(query)); // (keeps the address arithmetic below the key loop: its registers are all taken)
-        const bool ok = query < a.Lq;
-        const int64_t qrow = ok ? query : 0;
-        uint16_t *dqrow = const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + qrow * a.dq.ss;
-        uint16_t *dqbrow = nullptr;
-        if constexpr (C::NKR > 0) dqbrow = const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + qrow * a.dqb.ss;
-        // block n holds channels [32 n, 32 n + 32) of [dQ | dQ_b]; dQ_b starts at channel 16 NKD (a multiple
-        // of 16, so a 16-channel half of a block is all dq or all dq_bias)
-#pragma unroll
-        for (int n = 0; n < C::MB; ++n) {
-            if (32 * n + 32 <= 16 * C::NKD) {
-                store_acc_rows<T, C::VEC>(dqrow + 32 * n, ok, a.dq.vec_ok, acc[qb][n], a.scale, a.d - 32 * n, g);
-            } else if constexpr (C::NKR > 0) {
-                if (32 * n >= 16 * C::NKD) {
-                    const int cr = 32 * n - 16 * C::NKD;
-                    store_acc_rows<T, C::VEC>(dqbrow + cr, ok, a.dqb.vec_ok, acc[qb][n], 1.f, a.r - cr, g);
-                } else { // the block straddles: channels [32 n, 32 n + 16) are dq, the rest dq_bias
-                    f32x16_t lo, hi;
-#pragma unroll
-                    for (int v = 0; v < 8; ++v) {
-                        lo[v] = acc[qb][n][v];
-                        lo[8 + v] = 0.f;
-                        hi[v] = acc[qb][n][8 + v];
-                        hi[8 + v] = 0.f;
-                    }
-                    store_acc_rows<T, C::VEC>(dqrow + 32 * n, ok, a.dq.vec_ok, lo, a.scale, min(a.d - 32 * n, 16), g);
-                    store_acc_rows<T, C::VEC>(dqbrow, ok, a.dqb.vec_ok, hi, 1.f, min(a.r, 16), g);
-                }
-            } else {
-                store_acc_rows<T, C::VEC>(dqrow + 32 * n, ok, a.dq.vec_ok, acc[qb][n], a.scale, a.d - 32 * n, g);
-            }
-        }
+    // ---- epilogue of this batch entry: dq = scale * acc rows [0, d)
+    dq_store<T, C, false>(a, acc, b, h, wq0, c, g);
+    } // batch entries of the group
+
+    // ---- dq_bias = acc rows [16 NKD, 16 NKD + r), summed over the group's batch entries
+    if constexpr (C::NKR > 0) {
+        const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        dq_store<T, C, true>(a, acc, bg, h, wq0, lane_end & 31, lane_end >> 5);
     }
 }
 
@@ -495,7 +530,8 @@ static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
     static KernelOnce once;
     const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
     if (e != hipSuccess) return e;
-    const int64_t total = (int64_t)a.ntiles_m * a.B * a.H;
+    const int group = a.group > 1 ? a.group : 1;
+    const int64_t total = (int64_t)a.ntiles_m * ((a.B + group - 1) / group) * a.H;
     a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, once);
     return launch_flat(kern, total, C::NTHREADS, C::LDS_BYTES, stream, a);
 }

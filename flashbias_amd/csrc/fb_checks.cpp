@@ -64,6 +64,19 @@ size_t fb_bwd_workspace_bytes(const fb_params *p) {
     return fb::bwd_scratch_bytes((int64_t)p->B * p->H * p->Lq);
 }
 
+int fb_suggest_bias_grad_group(const fb_params *p) {
+    if (!p || p->r <= 0 || p->B < 32 || p->H <= 0 || p->Lq <= 0 || p->Lk <= 0) return 1;
+    if (p->q_bias.stride_b != 0 || p->k_bias.stride_b != 0) return 1;
+    // sequences of 1024 and more run kernels that keep one batch entry per workgroup
+    if (p->Lq >= 1024 || p->Lk >= 1024) return 1;
+    const int64_t lmin = p->Lq < p->Lk ? p->Lq : p->Lk;
+    // (measured on 4096 x 16 windows of 256 tokens: backward + reduction 5.34 ms ungrouped, 5.13 / 4.93 / 4.84 /
+    // 4.89 / 5.01 ms with groups of 2 / 4 / 8 / 16 / 32)
+    for (int g = 8; g > 1; g /= 2)
+        if (((int64_t)p->B + g - 1) / g * p->H * ((lmin + 255) / 256) >= 4096) return g;
+    return 1;
+}
+
 int fb_check(const fb_params *p, int pass) {
     g_err[0] = 0;
     if (!p) return fail(FB_ERR_NULL, "params: null pointer");
@@ -102,9 +115,13 @@ int fb_check(const fb_params *p, int pass) {
     if ((rc = check_out(p->dq, p->d, p->B, p->H, p->Lq, "dq"))) return rc;
     if ((rc = check_out(p->dk, p->d, p->B, p->H, p->Lk, "dk"))) return rc;
     if ((rc = check_out(p->dv, p->d, p->B, p->H, p->Lk, "dv"))) return rc;
+    if (p->bias_grad_group < 0) return fail(FB_ERR_SHAPE, "bias_grad_group must not be negative");
     if (p->r > 0) {
-        if ((rc = check_out(p->dq_bias, p->r, p->B, p->H, p->Lq, "dq_bias"))) return rc;
-        if ((rc = check_out(p->dk_bias, p->r, p->B, p->H, p->Lk, "dk_bias"))) return rc;
+        // with groups of g batch entries the factor gradients have ceil(B / g) batch rows
+        const int g = p->bias_grad_group > 1 ? p->bias_grad_group : 1;
+        const int rows = (int)(((int64_t)p->B + g - 1) / g);
+        if ((rc = check_out(p->dq_bias, p->r, rows, p->H, p->Lq, "dq_bias"))) return rc;
+        if ((rc = check_out(p->dk_bias, p->r, rows, p->H, p->Lk, "dk_bias"))) return rc;
     }
     if (!p->delta) return fail(FB_ERR_NULL, "%s: null pointer", "delta");
     if (reinterpret_cast<uintptr_t>(p->delta) % 16 != 0) return fail(FB_ERR_STRIDE, "%s: must be 16-byte aligned", "delta");

@@ -251,10 +251,17 @@ __device__ __forceinline__ void lds_dma16(const void *g, uint32_t lds) {
 // only the given lanes switched on.  All lanes of the wave must be active at the call.
 __device__ __forceinline__ void lds_dma16_lanes(uint32_t off, const void *base, uint32_t lds, uint64_t lanes) {
     uint64_t saved;
+    // (the base is wave-uniform by contract; said again here for pointers that run through nested loops, which the
+    // compiler may keep in vector registers: a scalar operand is what the instruction takes)
+    const uint64_t bb = reinterpret_cast<uint64_t>(base);
+    // (readfirstlane returns a signed int: each half goes through uint32_t, or a low half with its top bit set
+    // would sign-extend over the high half of the address)
+    const uint64_t ub = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(bb >> 32)) << 32) |
+                        (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)bb);
     asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %4\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\t"
                  "global_load_lds_dwordx4 %1, %2\n\ts_mov_b64 exec, %0"
                  : "=&s"(saved)
-                 : "v"(off), "s"(base), "s"(lds), "s"(lanes)
+                 : "v"(off), "s"(ub), "s"(lds), "s"(lanes)
                  : "memory");
 }
 __device__ __forceinline__ void lds_dma4(const void *g, uint32_t lds) {

@@ -36,6 +36,7 @@ struct BwdArgs {
     int slots;    // workgroups of this launch that share a compute unit (priority turn-taking)
     int stats_here; // dq kernel: compute -delta and lse * log2(e) itself (and store them) instead of reading them
     int stat_chunks; // writers of the scratch buffer: also store the statistics chunks (dkv_streamlined())
+    int group; // > 1: a workgroup serves this many consecutive batch entries and sums their factor gradients (row b / group)
 };
 
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.
@@ -83,7 +84,8 @@ inline bool dkv_streamlined(const BwdArgs &a) {
     const int64_t lim = (int64_t)1 << 24;
     return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
            (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.qb.ss < lim)) && a.q.ss < lim && a.dout.ss < lim &&
-           a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f && (a.Lq >= 1024 || small_grid(a.B, a.H, a.Lk));
+           a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f && (a.Lq >= 1024 || small_grid(a.B, a.H, a.Lk)) &&
+           a.group <= 1; // (factor gradients summed over groups of batch entries: the general kernels do that)
 }
 
 // The same for the streamlined dq kernel (fb_bwd_dq_lean.h), which streams K, K_b and V (general
@@ -95,7 +97,7 @@ inline bool dq_streamlined(const BwdArgs &a) {
     return a.mask.type == 0 && a.d == 32 && (a.r == 8 || a.r == 0) && a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok &&
            (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok && a.kb.ss < lim)) && a.k.ss < lim && a.v.ss < lim &&
            (!a.stats_here || a.o.vec_ok) && a.scale > 1e-6f && a.scale * 1.4426950408889634f <= 1.f &&
-           (a.Lk >= 2048 || small_grid(a.B, a.H, a.Lq));
+           (a.Lk >= 2048 || small_grid(a.B, a.H, a.Lq)) && a.group <= 1;
 }
 
 // What a launcher remembers about one kernel instantiation (one static object per instantiation;

@@ -159,8 +159,12 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
         p.dq = t4(dq); p.dk = t4(dk); p.dv = t4(dv);
         Tensor dqb_full, dkb_full;
         if (p.r) {
-            dqb_full = torch::empty({p.B, p.Lq, p.H, p.r}, q.options());
-            dkb_full = torch::empty({p.B, p.Lk, p.H, p.r}, q.options());
+            // factors shared by a large batch of short sequences: the kernels sum the gradients of `group` batch
+            // entries themselves and the full-shape tensors shrink by that factor
+            const int group = p.bias_grad_group = fb_suggest_bias_grad_group(&p);
+            const int64_t rows = ((int64_t)p.B + group - 1) / group;
+            dqb_full = torch::empty({rows, p.Lq, p.H, p.r}, q.options());
+            dkb_full = torch::empty({rows, p.Lk, p.H, p.r}, q.options());
             p.dq_bias = t4(dqb_full);
             p.dk_bias = t4(dkb_full);
         }

@@ -206,8 +206,12 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     p.dq, p.dk, p.dv = _tensor(dq), _tensor(dk), _tensor(dv)
     dqb_full = dkb_full = None
     if p.r:  # (also when only a folded vector mask makes up the factors)
-        dqb_full = torch.empty((p.B, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
-        dkb_full = torch.empty((p.B, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
+        # factors shared by a large batch of short sequences: the kernels sum the gradients of `group` batch
+        # entries themselves and the full-shape tensors shrink by that factor
+        group = p.bias_grad_group = lib.fb_suggest_bias_grad_group(p)
+        rows = -(-p.B // group)
+        dqb_full = torch.empty((rows, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
+        dkb_full = torch.empty((rows, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
         p.dq_bias, p.dk_bias = _tensor(dqb_full), _tensor(dkb_full)
     # scratch of the backward: -delta and lse * log2(e), sized by the library
     delta = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=lse.device, dtype=torch.float32)

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FB_VERSION 1
+#define FB_VERSION 2
 #define FB_MAX_HEADDIM 128 /* flash_bias_triton.py:1106 */
 #define FB_MAX_RANK 128
 /* Size of the library-owned scratch buffer used by fb_bwd_static (one copy per GPU, held until the
@@ -85,9 +85,16 @@ typedef struct fb_params {
     fb_tensor dout;             /* bwd in: upstream gradient of o */
     fb_tensor dq, dk, dv;       /* bwd out */
     fb_tensor dq_bias, dk_bias; /* bwd out, full (B, L, H, r) shape: the caller reduces over
-                                   broadcast dims */
+                                   broadcast dims (but see bias_grad_group) */
     float *delta;               /* backward scratch of fb_bwd_workspace_bytes() bytes, 16-byte aligned, written by the
                                    backward: -delta and lse * log2(e) per query row, as fp32 and as 16-bit parts */
+    int32_t bias_grad_group;    /* 0 or 1: as above.  g > 1, for factors that the batch shares (stride_b = 0, the
+                                   window attention of swin_transformer_v2.py:178-203): dq_bias and dk_bias have
+                                   ceil(B / g) batch rows and row i receives the sum of the gradients of batch
+                                   entries [i g, (i + 1) g), accumulated in fp32 inside the kernels and rounded
+                                   once; the caller reduces the remaining rows.  (The reference accumulates the factor
+                                   gradients with atomic adds into fp32 buffers laid out like the factors
+                                   themselves, flash_bias_triton.py:1219-1231, :1342.) */
 } fb_params;
 
 /* Library / ABI version. */
@@ -100,6 +107,14 @@ const char *fb_last_error(void);
  * (flash_bias_triton.py:1102-1129, :1201-1225) without touching the GPU.
  * pass: 0 = forward, 1 = backward. */
 int fb_check(const fb_params *p, int pass);
+
+/* The bias_grad_group this library recommends for a backward call: 1 unless both factors are shared by
+ * the batch (stride_b = 0) and the call is a large batch of short sequences (the window attention of
+ * swin_transformer_v2.py:178-203), where writing the full-shape factor gradients and summing them
+ * afterwards costs more than the attention itself saves; then the largest of 8, 4, 2 that still
+ * leaves every compute unit several workgroups.  Reads B, H, Lq, Lk, r and the factors' strides only.
+ * No counterpart in the reference. */
+int fb_suggest_bias_grad_group(const fb_params *p);
 
 /* Bytes of the backward's scratch buffer fb_params.delta for these sizes (24 per query row: two
  * floats and one 16-byte chunk of 16-bit parts, the second array starting on a 16-byte boundary;

@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fb_version() == 1
+    assert lib.fb_version() == 2
 
 
 def test_workspace_size_query():
@@ -101,6 +101,7 @@ def test_check_rejects_forward(mutate, code):
     (lambda p: setattr(p, "delta", None), -1),
     (lambda p: setattr(p.dk, "stride_h", 0), -4),
     (lambda p: setattr(p.dk_bias, "stride_b", 0), -4),
+    (lambda p: setattr(p, "bias_grad_group", -1), -2),
 ])
 def test_check_rejects_backward(mutate, code):
     p = _good(1)
@@ -109,6 +110,32 @@ def test_check_rejects_backward(mutate, code):
     assert lib.fb_check(p, 1) == code
     for fn in (lib.fb_bwd, lib.fb_bwd_preprocess, lib.fb_bwd_dkv, lib.fb_bwd_dq):
         assert fn(p, None) == code
+
+
+def test_grouped_factor_gradients_checks_and_suggestion():
+    """bias_grad_group = g: the factor gradients have ceil(B / g) batch rows, so a single group may
+    use a zero batch stride; the library suggests groups only for factors shared by a large batch of
+    short sequences."""
+    lib = _lib.load()
+    p = _good(1)
+    p.dq_bias.stride_b = p.dk_bias.stride_b = 0
+    assert lib.fb_check(p, 1) == -4          # two batch rows would alias
+    p.bias_grad_group = 2                    # one group of two: a single row
+    assert lib.fb_check(p, 1) == 0
+    assert lib.fb_suggest_bias_grad_group(p) == 1      # B = 2
+    p.B, p.H, p.Lq, p.Lk, p.r = 4096, 16, 256, 256, 16
+    assert lib.fb_suggest_bias_grad_group(p) == 1      # the factors are not shared by the batch
+    p.q_bias.stride_b = p.k_bias.stride_b = 0
+    assert lib.fb_suggest_bias_grad_group(p) == 8
+    p.B = 512
+    assert lib.fb_suggest_bias_grad_group(p) == 2      # still 4096 workgroups of 256 queries
+    p.B = 128
+    assert lib.fb_suggest_bias_grad_group(p) == 1
+    p.B, p.Lq = 4096, 1024
+    assert lib.fb_suggest_bias_grad_group(p) == 1      # long sequences keep one batch entry per workgroup
+    p.Lq, p.r = 256, 0
+    assert lib.fb_suggest_bias_grad_group(p) == 1
+    assert lib.fb_suggest_bias_grad_group(None) == 1
 
 
 @pytest.mark.parametrize("args,code", [

@@ -407,6 +407,113 @@ def test_backward_phases_through_the_c_abi(gpu_device):
     assert (parts[..., 6:] == 0).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,Lq,Lk,H,d,r,group,causal,mask", [
+    (11, 200, 200, 3, 32, 16, 4, False, False),   # ragged last group, window-sized sequences
+    (8, 256, 256, 2, 32, 8, 8, False, False),     # one group: a single row of factor gradients
+    (6, 130, 70, 2, 16, 16, 2, False, False),     # head dim 16: dq and dq_bias share an accumulator block
+    (5, 96, 96, 2, 64, 32, 3, True, False),
+    (4, 100, 100, 2, 24, 5, 2, False, False),     # unaligned rank: element-wise loaders and stores
+    (6, 64, 64, 4, 32, 16, 3, False, True)])      # additive matrix mask (the shifted windows of Swin)
+def test_factor_gradients_summed_over_batch_groups(gpu_device, dtype, B, Lq, Lk, H, d, r, group, causal, mask):
+    """fb_params.bias_grad_group = g: dq, dk, dv are those of the ungrouped call (bit for bit where both
+    run the same kernels), and row
+    i of dq_bias / dk_bias is the sum over batch entries [i g, (i + 1) g) of the ungrouped call's rows
+    (up to their 16-bit rounding: the grouped call rounds the fp32 sum once)."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _params, _stream, _tensor
+    dev = gpu_device
+    q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, Lq, Lk, H, d, r, dtype, seed=31)]
+    qb, kb = qb[:1], kb[:1]  # shared by the batch
+    m = None
+    if mask:
+        m = torch.where(torch.rand(1, 1, Lq, Lk, device=dev) < 0.2, -100.0, 0.0).to(dtype)
+    lib = _lib.load()
+
+    def run(g):
+        p, keep = _params(q, k, v, qb, kb, m, causal, None)
+        rows = -(-B // g)
+        bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, Lq), device=dev, dtype=torch.float32),
+                    dq=torch.empty_like(q), dk=torch.empty_like(k), dv=torch.empty_like(v),
+                    dqb=torch.full((rows, Lq, H, p.r), float("nan"), device=dev, dtype=dtype),
+                    dkb=torch.full((rows, Lk, H, p.r), float("nan"), device=dev, dtype=dtype),
+                    scratch=torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=dev, dtype=torch.float32))
+        p.o, p.lse, p.dout = _tensor(bufs["o"]), bufs["lse"].data_ptr(), _tensor(do)
+        p.dq, p.dk, p.dv = _tensor(bufs["dq"]), _tensor(bufs["dk"]), _tensor(bufs["dv"])
+        p.dq_bias, p.dk_bias, p.delta = _tensor(bufs["dqb"]), _tensor(bufs["dkb"]), bufs["scratch"].data_ptr()
+        p.bias_grad_group = g
+        _lib.check_status(lib.fb_fwd(p, _stream()))
+        _lib.check_status(lib.fb_bwd(p, _stream()))
+        torch.cuda.synchronize()
+        del keep
+        return bufs
+
+    one, grouped = run(1), run(group)
+    # head dim 32 with rank 8 runs the streamlined kernels ungrouped and the general ones grouped: equal
+    # up to rounding there, bit for bit everywhere else
+    same_kernels = not (d == 32 and r == 8)
+    for name in ("o", "lse", "dq", "dk", "dv"):
+        if same_kernels or name in ("o", "lse"):
+            assert torch.equal(one[name], grouped[name]), name
+        else:
+            a, b = one[name].float(), grouped[name].float()
+            assert (a - b).abs().max() <= 2e-2 * a.abs().max(), name
+    for name in ("dqb", "dkb"):
+        full = one[name].float()
+        pad = (-B) % group
+        if pad:
+            full = torch.cat([full, torch.zeros((pad,) + full.shape[1:], device=dev)])
+        want = full.view(-1, group, *full.shape[1:]).sum(1)
+        got = grouped[name].float()
+        assert torch.isfinite(got).all(), name
+        # the ungrouped rows carry one 16-bit rounding each, the grouped sum carries one in all
+        eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        tol = eps * (one[name].float().abs().view(-1, *full.shape[1:]).max() * group + want.abs().max())
+        assert (got - want).abs().max() <= tol, (name, float((got - want).abs().max()), float(tol))
+
+
+def test_shared_factors_large_batch_of_windows(gpu_device):
+    """A batch large enough for the library to suggest groups (64 windows x 16 heads of 256 tokens,
+    factors shared by the windows, as in swin_transformer_v2.py:178-203): all five gradients through
+    autograd against the oracle."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _params
+    dev = gpu_device
+    B, L, H, d, r = 512, 256, 16, 32, 16
+    q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=32)]
+    qb, kb = qb[:1].contiguous(), kb[:1].contiguous()
+    p, keep = _params(q, k, v, qb, kb, None, False, None)
+    assert _lib.load().fb_suggest_bias_grad_group(p) > 1
+    del keep
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, qb, kb)]
+    o = flash_bias_func(*leaves, None, False, None)
+    grads = torch.autograd.grad(o, leaves, do)
+    sub = slice(0, 8)  # o, dq, dk, dv of eight windows against the oracle
+    ref = oracle(q[sub], k[sub], v[sub], qb, kb, None, False, None, do[sub])
+    cpu = lambda t: t.detach().float().cpu()
+    assert (cpu(o[sub]) - ref[0]).abs().max() <= O_TOL[torch.bfloat16]
+    for name, got, want in zip(("dq", "dk", "dv"), grads[:3], ref[2:5]):
+        assert (cpu(got[sub]) - want).abs().max() <= GRAD_TOL * want.abs().max(), name
+    # the factor gradients: the sum over all windows, against the ungrouped path of the C ABI summed in fp64
+    from flashbias_amd.interface import _stream, _tensor
+    lib = _lib.load()
+    p, keep = _params(q, k, v, qb, kb, None, False, None)
+    lse = torch.empty((B, H, L), device=dev, dtype=torch.float32)
+    bufs = [torch.empty_like(q) for _ in range(4)]
+    full = [torch.empty((B, L, H, r), device=dev, dtype=q.dtype) for _ in range(2)]
+    scratch = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=dev, dtype=torch.float32)
+    p.o, p.lse, p.dout = _tensor(bufs[0]), lse.data_ptr(), _tensor(do)
+    p.dq, p.dk, p.dv = _tensor(bufs[1]), _tensor(bufs[2]), _tensor(bufs[3])
+    p.dq_bias, p.dk_bias, p.delta = _tensor(full[0]), _tensor(full[1]), scratch.data_ptr()
+    _lib.check_status(lib.fb_fwd(p, _stream()))
+    _lib.check_status(lib.fb_bwd(p, _stream()))
+    torch.cuda.synchronize()
+    for name, got, f in zip(("dq_bias", "dk_bias"), grads[3:], full):
+        want = f.double().sum(0, keepdim=True)
+        assert got.shape == want.shape
+        assert (got.double() - want).abs().max() <= 2e-2 * want.abs().max(), name
+
+
 @pytest.mark.parametrize("Lq,Lk", [(1000, 1000), (777, 1300), (1300, 777)])
 @pytest.mark.parametrize("causal", [False, True])
 def test_long_ragged_sequences(gpu_device, Lq, Lk, causal):
