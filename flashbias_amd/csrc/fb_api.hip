@@ -18,6 +18,8 @@ namespace fb {
 FB_DECL(bf16_1) FB_DECL(bf16_2) FB_DECL(bf16_4) FB_DECL(bf16_8)
 FB_DECL(f16_1) FB_DECL(f16_2) FB_DECL(f16_4) FB_DECL(f16_8)
 #undef FB_DECL
+hipError_t launch_bwd_both_bf16_2(const BwdArgs &a, hipStream_t stream);
+hipError_t launch_bwd_both_f16_2(const BwdArgs &a, hipStream_t stream);
 
 hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream) {
     switch (nkd_of(a.d)) {
@@ -44,6 +46,10 @@ hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream) {
     case 4: return bf16 ? launch_bwd_dq_bf16_4(a, stream) : launch_bwd_dq_f16_4(a, stream);
     default: return bf16 ? launch_bwd_dq_bf16_8(a, stream) : launch_bwd_dq_f16_8(a, stream);
     }
+}
+// dq and dk/dv workgroups of the streamlined kernels in one launch (fb_bwd_both.hip; head dim 32)
+hipError_t launch_bwd_both(const BwdArgs &a, bool bf16, hipStream_t stream) {
+    return bf16 ? launch_bwd_both_bf16_2(a, stream) : launch_bwd_both_f16_2(a, stream);
 }
 } // namespace fb
 
@@ -231,6 +237,14 @@ int fb_bwd(const fb_params *p, void *stream) {
     const int rc = fb_check(p, 1);
     if (rc) return rc;
     fb::BwdArgs a = bwd_args(p);
+    if (fb::mixed_backward(a)) {
+        // small grids of the streamlined kernels: the preprocess step, then one launch that holds the dq and
+        // the dk/dv workgroups side by side (same bits as the two launches)
+        const int rc1 = launched(fb::launch_bwd_preprocess(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                                 "fb_bwd_preprocess");
+        if (rc1) return rc1;
+        return launched(fb::launch_bwd_both(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd (dq + dk/dv)");
+    }
     a.stats_here = 1;
     const int rc2 = launched(fb::launch_bwd_dq(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd_dq");
     if (rc2) return rc2;

@@ -279,7 +279,7 @@ __device__ __forceinline__ void dkv_store(const BwdArgs &a, const f32x16_t (&acc
 }
 
 template <class T, class C>
-__device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
+__device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, int wg) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
 
@@ -293,7 +293,7 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
     const int group = a.group > 1 ? a.group : 1;
     const int nbg = (a.B + group - 1) / group;
     const int total = a.ntiles_n * nbg * a.H;
-    const int work = xcd_remap(blockIdx.x, total);
+    const int work = xcd_remap(wg, total);
     const int bgh = work / a.ntiles_n;
     const int tile_n = work % a.ntiles_n; // causal: low key tiles see the most queries, they go first
     const int bg = bgh / a.H, h = bgh % a.H;
@@ -587,7 +587,7 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a) {
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + 1))) void
 bwd_dkv_kernel(const BwdArgs a) {
-    bwd_dkv_body<T, C>(a);
+    bwd_dkv_body<T, C>(a, blockIdx.x);
 }
 
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART, bool FOLD>
@@ -664,11 +664,14 @@ static hipError_t launch_dkv_r(const BwdArgs &a, hipStream_t stream) {
     }
 }
 
-// Compiled once per (element type, head-dim bucket), see Makefile.
+// Compiled once per (element type, head-dim bucket), see Makefile.  (FB_BODIES_ONLY: included by the unit that
+// builds the mixed dq + dk/dv launch, which wants the kernels' bodies and not this entry point.)
+#ifndef FB_BODIES_ONLY
 #define FB_CAT2(a, b) a##b
 #define FB_CAT(a, b) FB_CAT2(a, b)
 hipError_t FB_CAT(launch_bwd_dkv_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
     return launch_dkv_r<FB_T, FB_NKD, FB_NDV>(a, stream);
 }
+#endif
 
 } // namespace fb

@@ -44,13 +44,16 @@ struct DkvLeanCfg {
 };
 
 template <class T, class C>
-__device__ __attribute__((noinline)) void dkv_lean_retry(const void *kernargs) {
+__device__ __attribute__((noinline)) void dkv_lean_retry(const void *kernargs, int wg) {
     const BwdArgs a = uniform_kernargs<BwdArgs>(kernargs);
-    bwd_dkv_body<T, typename C::General>(a);
+    bwd_dkv_body<T, typename C::General>(a, __builtin_amdgcn_readfirstlane(wg));
 }
 
+// The whole streamlined dk/dv computation of workgroup `wg` of the launch (the kernel below is nothing else; a
+// launch that mixes dq and dk/dv workgroups calls it with its own numbering).  `kernargs`: where the kernel's
+// argument block lives, for the out-of-line fallback.
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkv_lean_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, const void *kernargs) {
     constexpr int NKR = C::NKR;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -59,7 +62,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_n * a.B * a.H;
-    const int work = xcd_remap(blockIdx.x, total);
+    const int work = xcd_remap(wg, total);
     const int bh = work / a.ntiles_n;
     const int tile_n = work % a.ntiles_n; // causal: low key tiles see the most queries, they go first
     const int b = bh / a.H, h = bh % a.H;
@@ -94,7 +97,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         }
     }
     if (__syncthreads_or(bad)) {
-        dkv_lean_retry<T, C>((const void *)__builtin_amdgcn_kernarg_segment_ptr());
+        dkv_lean_retry<T, C>(kernargs, wg);
         return;
     }
     // ones against the parts of -lse * log2(e) (k-slots 0..2) and of -delta (k-slots 3..5)
@@ -353,6 +356,11 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     if constexpr (NKR > 0) // rows 0..7 of the third accumulator block (8..15 repeat them)
         store_acc_rows<T, true>(const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + krow * a.dkb.ss, ok, a.dkb.vec_ok,
                                 acc_dkb, 1.f, 8, g);
+}
+
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dkv_lean_kernel(const BwdArgs a) {
+    bwd_dkv_lean_body<T, C>(a, blockIdx.x, (const void *)__builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template <class T, int NKR>

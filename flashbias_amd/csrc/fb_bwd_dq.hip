@@ -204,7 +204,7 @@ __device__ __forceinline__ void dq_store(const BwdArgs &a, const f32x16_t (&acc)
 
 // The whole dq / dq_bias computation of one workgroup; the kernel below is nothing else.
 template <class T, class C>
-__device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
+__device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint16_t *stage0 = reinterpret_cast<uint16_t *>(smem);
 
@@ -218,7 +218,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
     const int group = a.group > 1 ? a.group : 1;
     const int nbg = (a.B + group - 1) / group;
     const int total = a.ntiles_m * nbg * a.H;
-    const int work = xcd_remap(blockIdx.x, total);
+    const int work = xcd_remap(wg, total);
     const int bgh = work / a.ntiles_m;
     int tile_m = work % a.ntiles_m;
     if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
@@ -518,7 +518,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a) {
 template <class T, class C>
 __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::QBLK == 1 && C::NK <= 3 ? 1 : 0)))) void
 bwd_dq_kernel(const BwdArgs a) {
-    bwd_dq_body<T, C>(a);
+    bwd_dq_body<T, C>(a, blockIdx.x);
 }
 
 template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2, bool FOLD, bool KB1 = false>
@@ -589,11 +589,14 @@ static hipError_t launch_dq_r(const BwdArgs &a, hipStream_t stream) {
     }
 }
 
-// Compiled once per (element type, head-dim bucket), see Makefile.
+// Compiled once per (element type, head-dim bucket), see Makefile.  (FB_BODIES_ONLY: included by the unit that
+// builds the mixed dq + dk/dv launch, which wants the kernels' bodies and not this entry point.)
+#ifndef FB_BODIES_ONLY
 #define FB_CAT2(a, b) a##b
 #define FB_CAT(a, b) FB_CAT2(a, b)
 hipError_t FB_CAT(launch_bwd_dq_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
     return launch_dq_r<FB_T, FB_NKD>(a, stream);
 }
+#endif
 
 } // namespace fb

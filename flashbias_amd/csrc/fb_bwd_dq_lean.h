@@ -40,13 +40,16 @@ struct DqLeanCfg {
 };
 
 template <class T, class C>
-__device__ __attribute__((noinline)) void dq_lean_retry(const void *kernargs) {
+__device__ __attribute__((noinline)) void dq_lean_retry(const void *kernargs, int wg) {
     const BwdArgs a = uniform_kernargs<BwdArgs>(kernargs);
-    bwd_dq_body<T, typename C::General>(a);
+    bwd_dq_body<T, typename C::General>(a, __builtin_amdgcn_readfirstlane(wg));
 }
 
+// The whole streamlined dq computation of workgroup `wg` of the launch (the kernel below is nothing else; a
+// launch that mixes dq and dk/dv workgroups calls it with its own numbering).  `kernargs`: where the kernel's
+// argument block lives, for the out-of-line fallback.
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_lean_kernel(const BwdArgs a) {
+__device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const void *kernargs) {
     constexpr int NKR = C::NKR;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -55,7 +58,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_m * a.B * a.H;
-    const int work = xcd_remap(blockIdx.x, total);
+    const int work = xcd_remap(wg, total);
     const int bh = work / a.ntiles_m;
     int tile_m = work % a.ntiles_m;
     if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
@@ -90,7 +93,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         }
     }
     if (__syncthreads_or(bad)) {
-        dq_lean_retry<T, C>((const void *)__builtin_amdgcn_kernarg_segment_ptr());
+        dq_lean_retry<T, C>(kernargs, wg);
         return;
     }
     // -lse * log2(e) and -delta of this lane's query
@@ -358,6 +361,11 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     if constexpr (NKR > 0) // rows 0..7 of the second accumulator block (8..15 repeat them)
         store_acc_rows<T, true>(const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + qrow * a.dqb.ss, ok, a.dqb.vec_ok,
                                 acc_dqb, 1.f, 8, g);
+}
+
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_dq_lean_kernel(const BwdArgs a) {
+    bwd_dq_lean_body<T, C>(a, blockIdx.x, (const void *)__builtin_amdgcn_kernarg_segment_ptr());
 }
 
 template <class T, int NKR>

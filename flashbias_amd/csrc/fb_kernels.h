@@ -100,6 +100,20 @@ inline bool dq_streamlined(const BwdArgs &a) {
            (a.Lk >= 2048 || small_grid(a.B, a.H, a.Lq)) && a.group <= 1;
 }
 
+// Whether fb_bwd runs the preprocess step and then one launch that mixes the streamlined dq and dk/dv workgroups
+// (fb_bwd_both.hip) instead of the dq and dk/dv launches: both streamlined kernels cover the call with the
+// statistics read from the scratch buffer, neither kind alone has more than one workgroup per compute unit
+// (measured at B2 H4, two launches against the mixed one: 0.035 / 0.021 ms at L=1024, 0.058 / 0.036 at 2048,
+// 0.112 / 0.096 at 4096, and 0.330 / 0.340 at 8192, where every SIMD has its two waves anyway), and both
+// kinds' workgroup counts split evenly over the eight XCDs (the mixed numbering alternates blocks of eight).
+inline bool mixed_backward(const BwdArgs &a0) {
+    BwdArgs a = a0;
+    a.stats_here = 0;
+    if (!(a.d == 32 && dq_streamlined(a) && dkv_streamlined(a))) return false;
+    const int64_t ndq = (int64_t)a.B * a.H * ((a.Lq + 127) / 128), ndkv = (int64_t)a.B * a.H * ((a.Lk + 127) / 128);
+    return ndq % 8 == 0 && ndkv % 8 == 0 && ndq <= num_cus() && ndkv <= num_cus();
+}
+
 // What a launcher remembers about one kernel instantiation (one static object per instantiation;
 // the only mutable state of the library besides num_cus() and fb_bwd_static's scratch address:
 // write-once values, atomics, so concurrent first calls from several threads are fine).

@@ -407,6 +407,55 @@ def test_backward_phases_through_the_c_abi(gpu_device):
     assert (parts[..., 6:] == 0).all()
 
 
+@pytest.mark.parametrize("dtype,B,H,Lq,Lk,r,causal", [
+    (torch.bfloat16, 2, 4, 1024, 1024, 8, False), (torch.float16, 2, 4, 2048, 2048, 8, True),
+    (torch.bfloat16, 2, 4, 4096, 4096, 0, False), (torch.bfloat16, 1, 8, 1000, 3000, 8, False),
+    (torch.bfloat16, 4, 2, 2500, 1111, 8, True)])
+def test_small_grid_backward_in_one_launch(gpu_device, dtype, B, H, Lq, Lk, r, causal):
+    """On grids that give neither backward kernel more than one workgroup per compute unit fb_bwd runs
+    the preprocess step and one launch that holds the dq and the dk/dv workgroups side by side: the
+    gradients and the scratch buffer are bit for bit those of the three phases launched one by one,
+    and the gradients pass the gate against the oracle (ragged and rectangular shapes included)."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _params, _stream, _tensor
+    dev = gpu_device
+    q, k, v, qb, kb, do = [None if t is None else t.to(dev) for t in make_inputs(B, Lq, Lk, H, 32, r, dtype, seed=41)]
+    do = do * 0.25
+    lib = _lib.load()
+
+    def params():
+        p, keep = _params(q, k, v, qb, kb, None, causal, None)
+        bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, Lq), device=dev, dtype=torch.float32),
+                    dq=torch.empty_like(q), dk=torch.empty_like(k), dv=torch.empty_like(v),
+                    scratch=torch.full((lib.fb_bwd_workspace_bytes(p) // 4,), float("nan"), device=dev,
+                                       dtype=torch.float32))
+        p.o, p.lse, p.dout = _tensor(bufs["o"]), bufs["lse"].data_ptr(), _tensor(do)
+        p.dq, p.dk, p.dv = _tensor(bufs["dq"]), _tensor(bufs["dk"]), _tensor(bufs["dv"])
+        if r:
+            bufs["dqb"] = torch.empty((B, Lq, H, r), device=dev, dtype=dtype)
+            bufs["dkb"] = torch.empty((B, Lk, H, r), device=dev, dtype=dtype)
+            p.dq_bias, p.dk_bias = _tensor(bufs["dqb"]), _tensor(bufs["dkb"])
+        p.delta = bufs["scratch"].data_ptr()
+        return p, keep, bufs
+
+    p1, keep1, whole = params()
+    _lib.check_status(lib.fb_fwd(p1, _stream()))
+    _lib.check_status(lib.fb_bwd(p1, _stream()))
+    p2, keep2, parts = params()
+    _lib.check_status(lib.fb_fwd(p2, _stream()))
+    for name in ("fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq"):
+        _lib.check_status(getattr(lib, name)(p2, _stream()))
+    torch.cuda.synchronize()
+    for name in whole:
+        assert torch.equal(whole[name], parts[name]), name
+    ref = oracle(q, k, v, qb, kb, None, causal, None, do)
+    cpu = lambda t: t.detach().float().cpu()
+    assert (cpu(whole["o"]) - ref[0]).abs().max() <= O_TOL[dtype]
+    names = ("dq", "dk", "dv") + (("dqb", "dkb") if r else ())
+    for name, want in zip(names, ref[2:]):
+        assert (cpu(whole[name]) - want).abs().max() <= GRAD_TOL * want.abs().max(), name
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("B,Lq,Lk,H,d,r,group,causal,mask", [
     (11, 200, 200, 3, 32, 16, 4, False, False),   # ragged last group, window-sized sequences
