@@ -129,7 +129,9 @@ int fb_fwd(const fb_params *p, void *stream);
 /* Replaces _flash_attn_backward (flash_bias_triton.py:1197-1342).  Two launches on the stream: the
  * query-stationary kernel (dq, dq_bias), which also forms delta = rowsum(o * dout) for its own
  * queries and leaves -delta and lse * log2(e) in the scratch buffer, then the key-stationary kernel
- * (dk, dv, dk_bias) that reads them.  The results are bit-identical to the three phases below
+ * (dk, dv, dk_bias) that reads them.  (On grids that would give each of these kernels at most one
+ * workgroup per compute unit: the preprocess phase, then a single launch that holds the workgroups of
+ * both kernels side by side.)  The results are bit-identical to the three phases below
  * called one by one.  Unlike the reference there is no fp32 dq_accum buffer, no
  * atomics and no final cast (:1212-1219, :1340-1342): dq and dq_bias are accumulated in
  * registers by a query-stationary kernel and written once, so every gradient is
