@@ -410,12 +410,14 @@ def test_backward_phases_through_the_c_abi(gpu_device):
 @pytest.mark.parametrize("dtype,B,H,Lq,Lk,r,causal", [
     (torch.bfloat16, 2, 4, 1024, 1024, 8, False), (torch.float16, 2, 4, 2048, 2048, 8, True),
     (torch.bfloat16, 2, 4, 4096, 4096, 0, False), (torch.bfloat16, 1, 8, 1000, 3000, 8, False),
-    (torch.bfloat16, 4, 2, 2500, 1111, 8, True)])
+    (torch.bfloat16, 4, 2, 2500, 1111, 8, True), (torch.float16, 2, 4, 1100, 1100, 8, False),
+    (torch.bfloat16, 1, 4, 640, 700, 0, False)])
 def test_small_grid_backward_in_one_launch(gpu_device, dtype, B, H, Lq, Lk, r, causal):
     """On grids that give neither backward kernel more than one workgroup per compute unit fb_bwd runs
     the preprocess step and one launch that holds the dq and the dk/dv workgroups side by side: the
     gradients and the scratch buffer are bit for bit those of the three phases launched one by one,
-    and the gradients pass the gate against the oracle (ragged and rectangular shapes included)."""
+    and the gradients pass the gate against the oracle (ragged and rectangular shapes, even and odd
+    tile counts included)."""
     from flashbias_amd import _lib
     from flashbias_amd.interface import _params, _stream, _tensor
     dev = gpu_device
