@@ -12,6 +12,7 @@ stream.  Differences from the reference, all on purpose:
 * ``softmax_scale`` of ``None`` or 0 gives ``1/sqrt(d)`` as in the reference (:1110).
 """
 import math
+import weakref
 
 import torch
 
@@ -70,6 +71,38 @@ def _fold_vector_mask(q, q_bias, k_bias, mask):
     return q_new, k_new
 
 
+#: bound on sum_c max_i |q_bias[i, c]| max_j |k_bias[j, c]| (an upper bound of every |bias_ij|) below which
+#: factors of rank < 8 are padded to rank 8: the kernels for rank 8 carry a bias term with a relative error of
+#: 2^-17, 0.002 in the logits at this bound.
+_SMALL_BIAS_BOUND = 256.0
+_bias_bound_cache = {}  # id(q_bias) -> (weakref(q_bias), weakref(k_bias), versions, bound)
+
+
+def _bias_terms_are_small(q_bias, k_bias):
+    """Whether the factors' entries are small enough for the rank-8 kernels (see _SMALL_BIAS_BOUND).
+    Decided on the host from two reductions on the device, i.e. with a synchronisation, so only for
+    leaf tensors (buffers, parameters, constants such as the geometry factors of a PDE solver: the
+    same objects call after call) and cached per tensor pair and version; while a graph is being
+    captured only the cache is consulted.  Everything else gets the conservative answer."""
+    if not (q_bias.is_leaf and k_bias.is_leaf):
+        return False
+    key = id(q_bias)
+    versions = (q_bias._version, k_bias._version)
+    hit = _bias_bound_cache.get(key)
+    if hit is not None and hit[0]() is q_bias and hit[1]() is k_bias and hit[2] == versions:
+        return hit[3] <= _SMALL_BIAS_BOUND
+    if torch.cuda.is_current_stream_capturing():
+        return False  # (a pair seen before the capture keeps its answer: that needs no synchronisation)
+    with torch.no_grad():
+        rank = q_bias.shape[-1]
+        bound = float((q_bias.detach().float().abs().reshape(-1, rank).amax(0)
+                       * k_bias.detach().float().abs().reshape(-1, rank).amax(0)).sum())
+    if len(_bias_bound_cache) > 64:
+        _bias_bound_cache.clear()
+    _bias_bound_cache[key] = (weakref.ref(q_bias), weakref.ref(k_bias), versions, bound)
+    return bound <= _SMALL_BIAS_BOUND
+
+
 def _prepare_factors(q, k, q_bias, k_bias, mask):
     """What the kernels get in place of (q_bias, k_bias, mask): a large vector mask folded into the
     factors, the rank zero-padded to a multiple of 8, the channel dimension contiguous.  Done once
@@ -95,8 +128,10 @@ def _prepare_factors(q, k, q_bias, k_bias, mask):
             # and a rank of 16 selects the kernels that keep the factors as they are and apply the
             # softmax scale to the fp32 accumulator.  The kernels that fold the scale into a 16-bit
             # operand (rank 8) carry every bias term with a relative error of 2^-17, which is 0.05 in
-            # the logits at |term| = 7000.
-            pad = (0, (16 if rank < 8 else -(-rank // 8) * 8) - rank)
+            # the logits at |term| = 7000.  Constant factors with small entries (a distance bias over
+            # points in a unit box) do take rank 8.
+            target = 8 if rank < 8 and _bias_terms_are_small(q_bias, k_bias) else (16 if rank < 8 else -(-rank // 8) * 8)
+            pad = (0, target - rank)
             q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
         # (padding a permuted view keeps its permuted layout)
         q_bias, k_bias = _last_dim_contiguous(q_bias), _last_dim_contiguous(k_bias)

@@ -757,6 +757,29 @@ def test_workload_pde(gpu_device):
     _run_workload(gpu_device, workloads.pde(N=2048), torch.bfloat16)
 
 
+def test_small_constant_factors_take_rank_8(gpu_device):
+    """Factors of rank below 8 are padded to 16 unless they are leaf tensors with small entries (the bound
+    on |bias| that the wrapper computes once per tensor pair): then to 8, which the streamlined kernels
+    take.  ALiBi's factors (entries in the thousands), factors computed on the fly and calls under
+    graph capture stay at 16."""
+    from flashbias_amd import interface as I
+    dev = gpu_device
+    w = workloads.pde(N=2048)
+    q, k = w["q"].to(dev), w["k"].to(dev)
+    qb, kb = w["q_bias"].to(dev), w["k_bias"].to(dev)
+    assert I._prepare_factors(q, k, qb, kb, None)[0].shape[-1] == 8
+    assert I._prepare_factors(q, k, qb, kb, None)[0].shape[-1] == 8          # (from the cache)
+    assert I._prepare_factors(q, k, qb * 1.0, kb * 1.0, None)[0].shape[-1] == 8  # new leaves: decided again
+    qg = qb.clone().requires_grad_(True)
+    assert I._prepare_factors(q, k, qg * 1.0, kb, None)[0].shape[-1] == 16   # not a leaf
+    qb.mul_(100.0)                                                           # in-place change: decided again
+    assert I._prepare_factors(q, k, qb, kb, None)[0].shape[-1] == 16
+    a = workloads.alibi(1024)
+    assert I._prepare_factors(a["q"].to(dev), a["k"].to(dev), a["q_bias"].to(dev), a["k_bias"].to(dev), None)[0].shape[-1] == 16
+    # the PDE workload with the streamlined kernels (rank 8), against the oracle
+    _run_workload(gpu_device, workloads.pde(N=4096), torch.bfloat16)
+
+
 def test_workload_pairformer(gpu_device):
     """Pairformer-shaped: rows as batch, rank-32 factors shared over rows (reduced N)."""
     _run_workload(gpu_device, workloads.pairformer(N=192), torch.bfloat16)
