@@ -54,9 +54,8 @@ static hipError_t launch_both_lean(const BwdArgs &a0, hipStream_t stream) {
     return launch_flat(kern, total, 256, lds, stream, a);
 }
 
-// Whether fb_bwd should run the mixed launch for this call (after the preprocess step): both
-// streamlined kernels cover it, the grid is small (either kernel alone would leave SIMDs with
-// one wave), and both kinds' workgroup counts split evenly over the eight XCDs.
+// Compiled once per element type for head dim 32 (see Makefile).  When fb_bwd takes this path is decided by
+// mixed_backward() in fb_kernels.h.
 #define FB_CAT2(a, b) a##b
 #define FB_CAT(a, b) FB_CAT2(a, b)
 hipError_t FB_CAT(launch_bwd_both_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
