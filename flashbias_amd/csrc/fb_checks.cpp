@@ -71,9 +71,11 @@ int fb_suggest_bias_grad_group(const fb_params *p) {
     if (p->Lq >= 1024 || p->Lk >= 1024) return 1;
     const int64_t lmin = p->Lq < p->Lk ? p->Lq : p->Lk;
     // (measured on 4096 x 16 windows of 256 tokens: backward + reduction 5.34 ms ungrouped, 5.13 / 4.93 / 4.84 /
-    // 4.89 / 5.01 ms with groups of 2 / 4 / 8 / 16 / 32)
+    // 4.89 / 5.01 ms with groups of 2 / 4 / 8 / 16 / 32; 768 rows x 4 heads of 768 tokens, rank 32: 1.76 ungrouped,
+    // 1.68 / 1.64 / 1.66 / 1.79 with 2 / 4 / 8 / 16; 1024 x 8 windows of 256: 0.735, 0.689 / 0.668 / 0.657 / 0.669:
+    // the largest group that leaves two 256-row workgroups per workgroup slot of the chip)
     for (int g = 8; g > 1; g /= 2)
-        if (((int64_t)p->B + g - 1) / g * p->H * ((lmin + 255) / 256) >= 4096) return g;
+        if (((int64_t)p->B + g - 1) / g * p->H * ((lmin + 255) / 256) >= 1024) return g;
     return 1;
 }
 

@@ -127,9 +127,9 @@ def test_grouped_factor_gradients_checks_and_suggestion():
     assert lib.fb_suggest_bias_grad_group(p) == 1      # the factors are not shared by the batch
     p.q_bias.stride_b = p.k_bias.stride_b = 0
     assert lib.fb_suggest_bias_grad_group(p) == 8
-    p.B = 512
-    assert lib.fb_suggest_bias_grad_group(p) == 2      # still 4096 workgroups of 256 queries
-    p.B = 128
+    p.B = 256
+    assert lib.fb_suggest_bias_grad_group(p) == 4      # still 1024 workgroups of 256 queries
+    p.B = 64
     assert lib.fb_suggest_bias_grad_group(p) == 1
     p.B, p.Lq = 4096, 1024
     assert lib.fb_suggest_bias_grad_group(p) == 1      # long sequences keep one batch entry per workgroup
