@@ -41,9 +41,11 @@ struct FwdCfg {
     static constexpr bool VEC = VEC_, MASK = MASK_, FOLD = FOLD_;
     static_assert(!FOLD_ || !MASK_, "the additive mask is not divided by the scale");
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
-    // query blocks (of 32) per wave: two where the registers allow, so that every key / value
-    // fragment read from LDS feeds two blocks and two waves per SIMD carry four softmax streams
-    static constexpr int QB = (QB2_ && NKD_ + NKR_ <= 3 && NDV_ == 1 && VEC_ && !MASK_) ? 2 : 1;
+    // query blocks (of 32) per wave: two where the registers allow (head dim <= 32, rank <= 32:
+    // 219-247 registers at four operand steps), so that every key / value fragment read from LDS
+    // feeds two blocks and two waves per SIMD carry four softmax streams (768 x 4 rows of 768
+    // tokens at rank 32: 0.77 -> 0.64 ms)
+    static constexpr int QB = (QB2_ && NKD_ + NKR_ <= 4 && NDV_ == 1 && VEC_ && !MASK_) ? 2 : 1;
     static constexpr int BM = NWAVES * 32 * QB;
     static constexpr int NK = NKD + NKR;
     // A wave computes KBLK * 32 keys at a time; an LDS tile (one barrier) holds SUBS such groups.
