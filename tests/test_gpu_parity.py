@@ -575,13 +575,15 @@ def test_long_ragged_sequences(gpu_device, Lq, Lk, causal):
 @pytest.mark.parametrize("B,H,Lq,Lk,r,causal", [(8, 16, 1000, 1000, 8, False), (8, 32, 700, 700, 8, True),
                                                  (4, 64, 777, 1300, 16, False), (8, 32, 1300, 777, 0, True),
                                                  (64, 16, 256, 256, 8, False), (64, 16, 128, 128, 16, False),
-                                                 (48, 16, 380, 300, 16, True)])
+                                                 (48, 16, 380, 300, 16, True),
+                                                 (16, 16, 700, 520, 32, False), (40, 16, 520, 700, 24, True)])
 def test_large_grids_ragged(gpu_device, B, H, Lq, Lk, r, causal):
     """Grids of at least two (causal: three) 256-query workgroups per compute unit of an MI355X
     (256 CUs): the launchers then pick the two-query-blocks-per-wave kernels, which the small
     cases above never reach; ragged last tiles, rectangular and causal shapes.  The last two are
     windows whose last 256-query workgroup would be half empty: they take 128-query workgroups on a
-    grid that would otherwise get the large ones."""
+    grid that would otherwise get the large ones.  Ranks 32 and 24: four operand steps per score, the
+    widest forward that keeps two query blocks per wave."""
     assert B * H * ((Lq + 255) // 256) >= (3 if causal else 2) * 256
     _case(gpu_device, B, Lq, Lk, H, 32, r, torch.bfloat16, causal, seed=13)
 
