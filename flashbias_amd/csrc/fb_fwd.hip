@@ -71,11 +71,13 @@ struct FwdCfg {
     static constexpr int K_PT = (K_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int KB_PT = (KB_TASKS + NTHREADS - 1) / NTHREADS;
     static constexpr int V_PT = (V_TASKS + NTHREADS - 1) / NTHREADS;
-    // registers: three waves per SIMD for the small configurations, one (512 registers) where the
+    // registers: three waves per SIMD for the configurations that need at most 168 (six operand steps
+    // with head dims up to 64: 158-166; the attribute is a cap the hardware honours, so a kernel that
+    // would fit three waves runs two unless it says three), one (512 registers) where the
     // mask values or an unaligned head dim of 128 would spill at 256, else two
     static constexpr bool BIG = (MASK_ && (NDV_ >= 2 || NKD_ + NKR_ >= 5)) || (!VEC_ && NDV_ == 4) ||
                                 2 * LDS_BYTES > 160 * 1024; // (one workgroup per CU anyway)
-    static constexpr int WAVES_EU = QB == 2 ? 2 : BIG ? 1 : (NK <= 4 && NDV <= 2) ? 3 : 2;
+    static constexpr int WAVES_EU = QB == 2 ? 2 : BIG ? 1 : (NK <= 6 && NDV <= 2) ? 3 : 2;
     // LDS fragments requested ahead of their use: all key steps of a group when they are few,
     // and the V^T fragments of a group when the head dimension is one MFMA block
     static constexpr int KPRE = NK <= 4 ? NK : 0;
