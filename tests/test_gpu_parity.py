@@ -5,6 +5,7 @@ Tolerances (the gate of the headline metric): max-abs error of o <= 1e-2 (fp16) 
 for each of dq, dk, dv, dq_bias, dk_bias: max|err| / max|ref| <= 5e-2; causal structure exact.
 """
 import math
+import os
 
 import pytest
 import torch
@@ -27,8 +28,9 @@ def _gate(got, ref, dtype, skip=()):
         err, rel = errors(g, w)
         if name == "o":
             assert err <= O_TOL[dtype], (name, err)
-        elif w.abs().max() == 0:  # e.g. a single visible key: dS is identically zero
-            assert err <= 1e-5, (name, err)
+        elif w.abs().max() == 0:  # e.g. a single visible key: dS is identically zero in exact arithmetic; here it is
+            # dP - delta, two fp32 sums of the same products in different orders, summed over the queries
+            assert err <= 1e-4, (name, err)
         elif name not in skip:
             assert rel <= GRAD_TOL, (name, err, rel)
 
@@ -586,6 +588,52 @@ def test_large_grids_ragged(gpu_device, B, H, Lq, Lk, r, causal):
     widest forward that keeps two query blocks per wave."""
     assert B * H * ((Lq + 255) // 256) >= (3 if causal else 2) * 256
     _case(gpu_device, B, Lq, Lk, H, 32, r, torch.bfloat16, causal, seed=13)
+
+
+def _random_configurations(n, seed):
+    """n configurations drawn with a fixed seed from everything the operator accepts: head dims 8 ... 128
+    (not only multiples of 8), ranks 0 ... 64, lengths 1 ... 900 on either side, either element type,
+    causal or not, broadcast factors, the three mask forms, explicit scales.  Sizes are chosen so that
+    some grids fill the chip (the launchers then pick their large-workgroup kernels) and most do not."""
+    import numpy as np
+    rng = np.random.RandomState(seed)
+    out = []
+    for i in range(n):
+        d = int(rng.choice([8, 16, 24, 32, 32, 32, 40, 64, 64, 96, 128]))
+        r = int(rng.choice([0, 2, 5, 8, 8, 16, 16, 24, 32, 64]))
+        big = rng.rand() < 0.25  # a grid of several workgroups per compute unit
+        B, H = (int(rng.randint(8, 25)), int(rng.choice([8, 16]))) if big else (int(rng.randint(1, 4)), int(rng.randint(1, 6)))
+        hi = 420 if big else 900
+        Lq, Lk = int(rng.randint(1, hi)), int(rng.randint(1, hi))
+        if d > 64 and big:
+            B = max(B // 4, 1)
+        causal = bool(rng.rand() < 0.4)
+        dtype = "bf16" if rng.rand() < 0.6 else "f16"
+        mask = str(rng.choice(["none", "none", "none", "vector", "matrix", "vector_f32"]))
+        bq = (bool(rng.rand() < 0.2), bool(rng.rand() < 0.2))
+        bk = (bool(rng.rand() < 0.2), bool(rng.rand() < 0.2))
+        scale = None if rng.rand() < 0.7 else float(rng.choice([1.0, 0.5, 0.05]))
+        out.append(pytest.param(B, H, Lq, Lk, d, r, causal, dtype, mask, bq, bk, scale, i,
+                                id="%d-B%dH%d-%dx%d-d%dr%d-%s%s-%s" % (i, B, H, Lq, Lk, d, r, dtype, "-causal" if causal else "", mask)))
+    return out
+
+
+# (FB_RANDOM_CASES / FB_RANDOM_SEED in the environment draw a longer or a different list for a soak run)
+@pytest.mark.parametrize("B,H,Lq,Lk,d,r,causal,dtype,mask_kind,bq,bk,scale,idx",
+                         _random_configurations(int(os.environ.get("FB_RANDOM_CASES", "36")),
+                                                int(os.environ.get("FB_RANDOM_SEED", "20240"))))
+def test_random_configurations(gpu_device, B, H, Lq, Lk, d, r, causal, dtype, mask_kind, bq, bk, scale, idx):
+    """Whatever the launchers choose for a configuration nobody picked by hand must meet the same gate."""
+    dt = torch.bfloat16 if dtype == "bf16" else torch.float16
+    g = torch.Generator().manual_seed(1000 + idx)
+    mask = None
+    if mask_kind == "vector":
+        mask = torch.randn(B, 1, 1, Lk, generator=g).to(dt)
+    elif mask_kind == "vector_f32":
+        mask = torch.randn(1, H, 1, Lk, generator=g)
+    elif mask_kind == "matrix":
+        mask = torch.randn(B, 1, Lq, Lk, generator=g).to(dt)
+    _case(gpu_device, B, Lq, Lk, H, d, r, dt, causal, mask=mask, scale=scale, seed=2000 + idx, bq=bq, bk=bk)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
