@@ -72,7 +72,9 @@ struct DkvCfg {
     // one wave per SIMD (512 registers) where two would spill: large head dims in one pass, and
     // masked instantiations beyond the smallest (they also hold a step's mask values)
     static constexpr bool BIG = MASK_ && PART_ == 0 && (NDV_ >= 2 || NKD_ + NKR_ >= 5);
-    static constexpr int WAVES_EU = BIG ? 1 : ((NK <= 8 && NDV <= 2) || PART_ != 0) ? 2 : 1;
+    // (aligned, unmasked, at most four operand steps, head dim <= 32: 164-168 registers, and the third wave is worth
+    // more than the few that the allocator would otherwise take beyond 168)
+    static constexpr int WAVES_EU = BIG ? 1 : (VEC_ && !MASK_ && PART_ == 0 && NK <= 4 && NDV == 1) ? 3 : ((NK <= 8 && NDV <= 2) || PART_ != 0) ? 2 : 1;
 };
 
 template <class C>
@@ -317,6 +319,9 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, int wg) {
             for (int n = 0; n < (C::DO_DK ? C::MB1 - C::MB0 : 1); ++n) acc_dk[kb][n][v] = 0.f;
         }
 
+    // the key-side factor operand outlives a batch entry when the batch shares the factor (stride 0)
+    u32x4_t kbreg[C::KBW][C::NKR > 0 ? C::NKR : 1];
+
     for (int bi = 0; bi < group; ++bi) {
     const int b = __builtin_amdgcn_readfirstlane(bg * group + bi); // (wave-uniform, and the compiler should know)
     if (b >= a.B) break;
@@ -357,9 +362,13 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, int wg) {
             if (t < C::NKD)
                 kreg[kb][t] = load_chunk<C::VEC>(kbase, a.k.ss, key, a.Lk, 16 * t + 8 * g, a.d);
             else if constexpr (C::NKR > 0) {
-                const bool low = C::low_parts(a) && g == 1;
-                kreg[kb][t] = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, low ? 0 : 16 * (t - C::NKD) + 8 * g, a.r);
-                if (C::FOLD && a.scale != 1.f) kreg[kb][t] = fold_scale_chunk<T>(kreg[kb][t], 1.f / a.scale, C::low_parts(a), low);
+                u32x4_t &keep = kbreg[kb][t - C::NKD];
+                if (bi == 0 || a.kb.sb != 0) {
+                    const bool low = C::low_parts(a) && g == 1;
+                    keep = load_chunk<C::VEC>(kbbase, a.kb.ss, key, a.Lk, low ? 0 : 16 * (t - C::NKD) + 8 * g, a.r);
+                    if (C::FOLD && a.scale != 1.f) keep = fold_scale_chunk<T>(keep, 1.f / a.scale, C::low_parts(a), low);
+                }
+                kreg[kb][t] = keep;
             }
         }
         if constexpr (C::DO_DK) {

@@ -240,6 +240,8 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[qb][n][v] = 0.f;
     int turn = __builtin_amdgcn_readfirstlane(cu_slot());
+    // the query-side factor operand outlives a batch entry when the batch shares the factor (stride 0)
+    u32x4_t qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
 
     for (int bi = 0; bi < group; ++bi) {
     const int b = __builtin_amdgcn_readfirstlane(bg * group + bi); // (wave-uniform, and the compiler should know)
@@ -266,7 +268,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
                 (b * a.mask.sb + h * a.mask.sh) * (a.mask.is_f32 ? 4 : 2);
 
     // ---- query-side operands, resident in registers
-    u32x4_t qr[C::QBLK][C::NKD], qbr[C::QBLK][C::NKR > 0 ? C::NKR : 1];
+    u32x4_t qr[C::QBLK][C::NKD];
     u32x4_t dor[C::QBLK][C::NKD];
     float lse2[C::QBLK]; // lse * log2(e) of this lane's queries
     // -delta of this lane's query in all 16 registers of an accumulator block: the initial value
@@ -281,11 +283,13 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
             dor[qb][t] = load_chunk<C::VEC>(dobase, a.dout.ss, query, a.Lq, 16 * t + 8 * g, a.d);
         }
         if constexpr (C::NKR > 0) {
+            if (bi == 0 || a.qb.sb != 0) {
 #pragma unroll
-            for (int t = 0; t < C::NKR; ++t) {
-                const bool low = C::low_parts(a) && g == 1;
-                qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, low ? 0 : 16 * t + 8 * g, a.r);
-                if (C::FOLD && a.scale != 1.f) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, C::low_parts(a), low);
+                for (int t = 0; t < C::NKR; ++t) {
+                    const bool low = C::low_parts(a) && g == 1;
+                    qbr[qb][t] = load_chunk<C::VEC>(qbbase, a.qb.ss, query, a.Lq, low ? 0 : 16 * t + 8 * g, a.r);
+                    if (C::FOLD && a.scale != 1.f) qbr[qb][t] = fold_scale_chunk<T>(qbr[qb][t], 1.f / a.scale, C::low_parts(a), low);
+                }
             }
         }
         const bool ok = query < a.Lq;
@@ -518,7 +522,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
 // (One query block per wave and at most four operand steps fit 168 registers: a third wave per SIMD, which the
 // upper bound of the attribute has to allow; 768 x 4 rows of 768 tokens at rank 32: 0.80 -> 0.71 ms.)
 template <class T, class C>
-__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU, C::WAVES_EU + (C::QBLK == 1 && C::NK <= 4 ? 1 : 0)))) void
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(C::WAVES_EU + (C::QBLK == 1 && C::NK <= 4 && C::VEC && !C::MASK ? 1 : 0), C::WAVES_EU + (C::QBLK == 1 && C::NK <= 4 ? 1 : 0)))) void
 bwd_dq_kernel(const BwdArgs a) {
     bwd_dq_body<T, C>(a, blockIdx.x);
 }
