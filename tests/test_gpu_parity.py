@@ -17,7 +17,10 @@ pytestmark = pytest.mark.gpu
 NAMES = ("o", "dq", "dk", "dv", "dq_bias", "dk_bias")
 
 
-def _gate(got, ref, dtype, skip=()):
+def _gate(got, ref, dtype, skip=(), o_by_magnitude=False):
+    """o_by_magnitude: the tolerance on o (an absolute one, stated for benchmark-like inputs whose outputs stay
+    below 2) grows with max|o| beyond 2: under a peaked softmax o is close to single rows of v, |o| reaches 4-5,
+    and rounding the output to bf16 alone costs up to 2^-6 there."""
     refs = [ref[0]] + list(ref[2:])
     for name, g, w in zip(NAMES, got, refs):
         if w is None:
@@ -27,7 +30,8 @@ def _gate(got, ref, dtype, skip=()):
         assert torch.isfinite(g).all(), name
         err, rel = errors(g, w)
         if name == "o":
-            assert err <= O_TOL[dtype], (name, err)
+            tol = O_TOL[dtype] * (max(1.0, float(w.abs().max()) / 2.0) if o_by_magnitude else 1.0)
+            assert err <= tol, (name, err, tol)
         elif w.abs().max() == 0:  # e.g. a single visible key: dS is identically zero in exact arithmetic; here it is
             # dP - delta, two fp32 sums of the same products in different orders, summed over the queries
             assert err <= 1e-4, (name, err)
@@ -35,11 +39,11 @@ def _gate(got, ref, dtype, skip=()):
             assert rel <= GRAD_TOL, (name, err, rel)
 
 
-def _case(gpu_device, B, Lq, Lk, H, d, r, dtype, causal, mask=None, scale=None, seed=1, **bc):
+def _case(gpu_device, B, Lq, Lk, H, d, r, dtype, causal, mask=None, scale=None, seed=1, o_by_magnitude=False, **bc):
     q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, dtype, seed=seed, **bc)
     ref = oracle(q, k, v, qb, kb, mask, causal, scale, do)
     got = run_gpu(flash_bias_func, q, k, v, qb, kb, mask, causal, scale, do, gpu_device)
-    _gate(got, ref, dtype)
+    _gate(got, ref, dtype, o_by_magnitude=o_by_magnitude)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -633,7 +637,8 @@ def test_random_configurations(gpu_device, B, H, Lq, Lk, d, r, causal, dtype, ma
         mask = torch.randn(1, H, 1, Lk, generator=g)
     elif mask_kind == "matrix":
         mask = torch.randn(B, 1, Lq, Lk, generator=g).to(dt)
-    _case(gpu_device, B, Lq, Lk, H, d, r, dt, causal, mask=mask, scale=scale, seed=2000 + idx, bq=bq, bk=bk)
+    # (explicit scales of 0.5 and 1 give logits with a spread of 4-11: peaked rows, outputs as large as v itself)
+    _case(gpu_device, B, Lq, Lk, H, d, r, dt, causal, mask=mask, scale=scale, seed=2000 + idx, o_by_magnitude=True, bq=bq, bk=bk)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
