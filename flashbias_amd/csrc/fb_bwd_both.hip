@@ -16,7 +16,7 @@
 
 namespace fb {
 
-template <class T, int NKR>
+template <class T, int NKR, bool BG>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_both_lean_kernel(const BwdArgs a) {
     const void *kernargs = (const void *)__builtin_amdgcn_kernarg_segment_ptr();
     const int ndq = a.ntiles_m * a.B * a.H, ndkv = a.ntiles_n * a.B * a.H;
@@ -33,20 +33,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         wg = id - paired;
     }
     if (is_dq)
-        bwd_dq_lean_body<T, DqLeanCfg<T, NKR>>(a, wg, kernargs);
+        bwd_dq_lean_body<T, DqLeanCfg<T, NKR, BG>>(a, wg, kernargs);
     else
-        bwd_dkv_lean_body<T, DkvLeanCfg<T, NKR>>(a, wg, kernargs);
+        bwd_dkv_lean_body<T, DkvLeanCfg<T, NKR, BG>>(a, wg, kernargs);
 }
 
-template <class T, int NKR>
+template <class T, int NKR, bool BG = true>
 static hipError_t launch_both_lean(const BwdArgs &a0, hipStream_t stream) {
-    typedef DqLeanCfg<T, NKR> Cq;
-    typedef DkvLeanCfg<T, NKR> Ck;
+    typedef DqLeanCfg<T, NKR, BG> Cq;
+    typedef DkvLeanCfg<T, NKR, BG> Ck;
     BwdArgs a = a0;
     a.ntiles_m = (a.Lq + Cq::BM - 1) / Cq::BM;
     a.ntiles_n = (a.Lk + Ck::BN - 1) / Ck::BN;
     constexpr int lds = Cq::LDS_BYTES > Ck::LDS_BYTES ? Cq::LDS_BYTES : Ck::LDS_BYTES;
-    auto kern = bwd_both_lean_kernel<T, NKR>;
+    auto kern = bwd_both_lean_kernel<T, NKR, BG>;
     static KernelOnce once;
     const hipError_t e = allow_lds(kern, lds, once);
     if (e != hipSuccess) return e;
@@ -59,7 +59,8 @@ static hipError_t launch_both_lean(const BwdArgs &a0, hipStream_t stream) {
 #define FB_CAT2(a, b) a##b
 #define FB_CAT(a, b) FB_CAT2(a, b)
 hipError_t FB_CAT(launch_bwd_both_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
-    return a.r == 0 ? launch_both_lean<FB_T, 0>(a, stream) : launch_both_lean<FB_T, 1>(a, stream);
+    if (a.r == 0) return launch_both_lean<FB_T, 0>(a, stream);
+    return a.dqb.ptr ? launch_both_lean<FB_T, 1>(a, stream) : launch_both_lean<FB_T, 1, false>(a, stream);
 }
 
 } // namespace fb

@@ -588,8 +588,10 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, int wg) {
 
     // ---- dk_bias, summed over the group's batch entries
     if constexpr (C::NKR > 0 && C::DO_DK) {
-        const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-        dkv_store<T, C, true>(a, acc_dv, acc_dk, bg, h, wk0, lane_end & 31, lane_end >> 5);
+        if (a.dkb.ptr) { // (null: the caller does not want the factor gradients)
+            const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            dkv_store<T, C, true>(a, acc_dv, acc_dk, bg, h, wk0, lane_end & 31, lane_end >> 5);
+        }
     }
 }
 
@@ -653,7 +655,12 @@ static hipError_t launch_dkv_cfg(const BwdArgs &a, hipStream_t stream) {
         // the streamlined kernel: same 128-key workgroups as the general one, and ahead of it at every
         // grid size (measured at B2 H4: 0.019 against 0.023 ms at L=1024, 0.063 against 0.082 at 4096,
         // 0.73 against 0.82 at 16384)
-        if (dkv_streamlined(a)) return launch_dkv_lean<T, NKR>(a, stream);
+        if (dkv_streamlined(a)) {
+            if constexpr (NKR > 0) {
+                if (!a.dkb.ptr) return launch_dkv_lean<T, NKR, false>(a, stream);
+            }
+            return launch_dkv_lean<T, NKR>(a, stream);
+        }
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lq)) return launch_dkv_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);

@@ -24,9 +24,12 @@
 
 namespace fb {
 
-template <class T, int NKR_>
+// BG_: also accumulate and store dk_bias (false: the caller does not want the factor gradients, and the block
+// step keeps its slots but two of them carry no MFMA and no transposing read).
+template <class T, int NKR_, bool BG_ = true>
 struct DkvLeanCfg {
     static constexpr int NKR = NKR_;
+    static constexpr bool BG = BG_ && NKR_ > 0;
     static_assert(NKR_ <= 1, "rank 8 or none");
     static constexpr int NWAVES = 4, NTHREADS = 256, BN = 128, BM = 64;
     static constexpr int Q_BYTES = BM * 64, B_BYTES = BM * 32, AUX_BYTES = BM * 16, DO_BYTES = BM * 64;
@@ -207,7 +210,7 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
     auto read_col_d = [&](int qb, int t) { cd = lds_load_tr(tq[0] + C::DO_OFF + (2 * qb + t) * 1024, tq[1] + C::DO_OFF + (2 * qb + t) * 1024); };
     auto read_col_q = [&](int qb, int t) { cq4 = lds_load_tr(tq[0] + (2 * qb + t) * 1024, tq[1] + (2 * qb + t) * 1024); };
     auto read_col_b = [&](int qb, int t) {
-        if constexpr (NKR > 0) cqb = lds_load_tr(tb[t][0] + qb * 1024, tb[t][1] + qb * 1024);
+        if constexpr (C::BG) cqb = lds_load_tr(tb[t][0] + qb * 1024, tb[t][1] + qb * 1024);
     };
     const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // -inf (p = 0) for queries past the end and pairs that a causal mask hides
@@ -273,7 +276,7 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
         sn = T::mfma(fq[1], kr[1], sn);
         v4(0, 12, pp0, pds0);
         FB_SLOT_END;
-        if constexpr (NKR > 0) mfma_into<T>(acc_dkb, cqb, pds1);
+        if constexpr (C::BG) mfma_into<T>(acc_dkb, cqb, pds1);
         read_col_b(qb, 0);
         v4(0, 16, pp0, pds0);
         FB_SLOT_END;
@@ -296,7 +299,7 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
         v4(1, 12, pp1, pds1);
         read_rows_aux(qb);
         FB_SLOT_END;
-        if constexpr (NKR > 0) mfma_into<T>(acc_dkb, cqb, pds0);
+        if constexpr (C::BG) mfma_into<T>(acc_dkb, cqb, pds0);
         read_col_b(qb, 1);
         v4(1, 16, pp1, pds1);
         FB_SLOT_END;
@@ -338,12 +341,12 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
     // the second half of the last block
     mfma_into<T>(acc_dv, cd, pp1);
     mfma_into<T>(acc_dk, cq4, pds1);
-    if constexpr (NKR > 0) mfma_into<T>(acc_dkb, cqb, pds1);
+    if constexpr (C::BG) mfma_into<T>(acc_dkb, cqb, pds1);
 #undef FB_SLOT_END
 
     // ---- epilogue: dv, dk (times scale), dk_bias of this lane's key.  (The wait states let the
     // last accumulating MFMAs, which the compiler does not see as such, finish writing.)
-    if constexpr (NKR > 0)
+    if constexpr (C::BG)
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dv), "+v"(acc_dk), "+v"(acc_dkb));
     else
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dv), "+v"(acc_dk));
@@ -353,7 +356,7 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
                             32, g);
     store_acc_rows<T, true>(const_cast<uint16_t *>(a.dk.ptr) + b * a.dk.sb + h * a.dk.sh + krow * a.dk.ss, ok, a.dk.vec_ok, acc_dk,
                             a.scale, 32, g);
-    if constexpr (NKR > 0) // rows 0..7 of the third accumulator block (8..15 repeat them)
+    if constexpr (C::BG) // rows 0..7 of the third accumulator block (8..15 repeat them)
         store_acc_rows<T, true>(const_cast<uint16_t *>(a.dkb.ptr) + b * a.dkb.sb + h * a.dkb.sh + krow * a.dkb.ss, ok, a.dkb.vec_ok,
                                 acc_dkb, 1.f, 8, g);
 }
@@ -363,9 +366,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     bwd_dkv_lean_body<T, C>(a, blockIdx.x, (const void *)__builtin_amdgcn_kernarg_segment_ptr());
 }
 
-template <class T, int NKR>
+template <class T, int NKR, bool BG = true>
 static hipError_t launch_dkv_lean(const BwdArgs &a0, hipStream_t stream) {
-    typedef DkvLeanCfg<T, NKR> C;
+    typedef DkvLeanCfg<T, NKR, BG> C;
     BwdArgs a = a0;
     a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
     auto kern = bwd_dkv_lean_kernel<T, C>;

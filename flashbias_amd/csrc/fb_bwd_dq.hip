@@ -514,8 +514,10 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
 
     // ---- dq_bias = acc rows [16 NKD, 16 NKD + r), summed over the group's batch entries
     if constexpr (C::NKR > 0) {
-        const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-        dq_store<T, C, true>(a, acc, bg, h, wq0, lane_end & 31, lane_end >> 5);
+        if (a.dqb.ptr) { // (null: the caller does not want the factor gradients)
+            const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            dq_store<T, C, true>(a, acc, bg, h, wq0, lane_end & 31, lane_end >> 5);
+        }
     }
 }
 
@@ -576,7 +578,12 @@ static hipError_t launch_dq_cfg(const BwdArgs &a, hipStream_t stream) {
     if (a.mask.type)
         return vec ? launch_dq_vec<T, NKD, NKR, true, true>(a, stream) : launch_dq_vec<T, NKD, NKR, false, true>(a, stream);
     if constexpr (NKD == 2 && NKR <= 1) {
-        if (dq_streamlined(a)) return launch_dq_lean<T, NKR>(a, stream);
+        if (dq_streamlined(a)) {
+            if constexpr (NKR > 0) {
+                if (!a.dqb.ptr) return launch_dq_lean<T, NKR, false>(a, stream);
+            }
+            return launch_dq_lean<T, NKR>(a, stream);
+        }
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_dq_vec<T, NKD, NKR, true, false, true>(a, stream);

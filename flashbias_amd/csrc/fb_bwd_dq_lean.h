@@ -22,9 +22,11 @@
 
 namespace fb {
 
-template <class T, int NKR_>
+// BG_: also accumulate and store dq_bias (false: the caller does not want the factor gradients).
+template <class T, int NKR_, bool BG_ = true>
 struct DqLeanCfg {
     static constexpr int NKR = NKR_;
+    static constexpr bool BG = BG_ && NKR_ > 0;
     static_assert(NKR_ <= 1, "rank 8 or none");
     static constexpr int NWAVES = 4, NTHREADS = 256, BM = 128, BN = 64;
     static constexpr int K_BYTES = BN * 64, B_BYTES = BN * 32, V_BYTES = BN * 64;
@@ -230,7 +232,7 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
     };
     auto read_col_k = [&](int kb, int t) { ck = lds_load_tr(tq[0] + (2 * kb + t) * 1024, tq[1] + (2 * kb + t) * 1024); };
     auto read_col_b = [&](int kb, int t) {
-        if constexpr (NKR > 0) ckb = lds_load_tr(tb[t][0] + kb * 1024, tb[t][1] + kb * 1024);
+        if constexpr (C::BG) ckb = lds_load_tr(tb[t][0] + kb * 1024, tb[t][1] + kb * 1024);
     };
     // -inf (p = 0) for keys past the end and pairs that a causal mask hides
     auto hide = [&](f32x16_t &s, int k0) {
@@ -289,7 +291,7 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
         sn = T::mfma(fk[1], qr[1], sn);
         v4(0, 8, 4, pds0);
         FB_SLOT_END;
-        if constexpr (NKR > 0) mfma_into<T>(acc_dqb, ckb, pds1);
+        if constexpr (C::BG) mfma_into<T>(acc_dqb, ckb, pds1);
         read_col_b(kb, 0);
         v4(0, 12, 4, pds0);
         FB_SLOT_END;
@@ -308,7 +310,7 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
         v4(1, 8, 4, pds1);
         read_rows_v(kb);
         FB_SLOT_END;
-        if constexpr (NKR > 0) mfma_into<T>(acc_dqb, ckb, pds0);
+        if constexpr (C::BG) mfma_into<T>(acc_dqb, ckb, pds0);
         read_col_b(kb, 1);
         v4(1, 12, 8, pds1);
         FB_SLOT_END;
@@ -346,19 +348,19 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
     // the second half of the last block (two wait states after its conversion)
     asm volatile("s_nop 1" : "+v"(pds1));
     mfma_into<T>(acc_dq, ck, pds1);
-    if constexpr (NKR > 0) mfma_into<T>(acc_dqb, ckb, pds1);
+    if constexpr (C::BG) mfma_into<T>(acc_dqb, ckb, pds1);
 #undef FB_SLOT_END
 
     // ---- epilogue: dq (times scale) and dq_bias of this lane's query.  (The wait states let the
     // last accumulating MFMAs, which the compiler does not see as such, finish writing.)
-    if constexpr (NKR > 0)
+    if constexpr (C::BG)
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dq), "+v"(acc_dqb));
     else
         asm volatile("s_nop 15\n\ts_nop 15" : "+v"(acc_dq));
     const int64_t qrow = ok ? query : 0;
     store_acc_rows<T, true>(const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + qrow * a.dq.ss, ok, a.dq.vec_ok, acc_dq,
                             a.scale, 32, g);
-    if constexpr (NKR > 0) // rows 0..7 of the second accumulator block (8..15 repeat them)
+    if constexpr (C::BG) // rows 0..7 of the second accumulator block (8..15 repeat them)
         store_acc_rows<T, true>(const_cast<uint16_t *>(a.dqb.ptr) + b * a.dqb.sb + h * a.dqb.sh + qrow * a.dqb.ss, ok, a.dqb.vec_ok,
                                 acc_dqb, 1.f, 8, g);
 }
@@ -368,9 +370,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     bwd_dq_lean_body<T, C>(a, blockIdx.x, (const void *)__builtin_amdgcn_kernarg_segment_ptr());
 }
 
-template <class T, int NKR>
+template <class T, int NKR, bool BG = true>
 static hipError_t launch_dq_lean(const BwdArgs &a0, hipStream_t stream) {
-    typedef DqLeanCfg<T, NKR> C;
+    typedef DqLeanCfg<T, NKR, BG> C;
     BwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = bwd_dq_lean_kernel<T, C>;

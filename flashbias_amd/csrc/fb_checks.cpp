@@ -122,8 +122,11 @@ int fb_check(const fb_params *p, int pass) {
         // with groups of g batch entries the factor gradients have ceil(B / g) batch rows
         const int g = p->bias_grad_group > 1 ? p->bias_grad_group : 1;
         const int rows = (int)(((int64_t)p->B + g - 1) / g);
-        if ((rc = check_out(p->dq_bias, p->r, rows, p->H, p->Lq, "dq_bias"))) return rc;
-        if ((rc = check_out(p->dk_bias, p->r, rows, p->H, p->Lk, "dk_bias"))) return rc;
+        // both pointers null: the caller does not want the factor gradients (constant factors)
+        if (p->dq_bias.ptr || p->dk_bias.ptr) {
+            if ((rc = check_out(p->dq_bias, p->r, rows, p->H, p->Lq, "dq_bias"))) return rc;
+            if ((rc = check_out(p->dk_bias, p->r, rows, p->H, p->Lk, "dk_bias"))) return rc;
+        }
     }
     if (!p->delta) return fail(FB_ERR_NULL, "%s: null pointer", "delta");
     if (reinterpret_cast<uintptr_t>(p->delta) % 16 != 0) return fail(FB_ERR_STRIDE, "%s: must be 16-byte aligned", "delta");

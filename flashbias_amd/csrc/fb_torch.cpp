@@ -158,10 +158,13 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
         p.dout = t4(dout);
         p.dq = t4(dq); p.dk = t4(dk); p.dv = t4(dv);
         Tensor dqb_full, dkb_full;
-        if (p.r) {
-            // factors shared by a large batch of short sequences: the kernels sum the gradients of `group` batch
-            // entries themselves and the full-shape tensors shrink by that factor
-            const int group = p.bias_grad_group = fb_suggest_bias_grad_group(&p);
+        // (neither factor asks for its gradient: constant factors; the library then skips them)
+        const bool factor_grads = p.r && (ctx->needs_input_grad(3) || ctx->needs_input_grad(4));
+        // factors shared by a large batch of short sequences: a workgroup walks `group` batch entries (it then loads
+        // the factor operand it keeps once), sums their factor gradients itself, and the full-shape tensors shrink by
+        // that factor
+        const int group = p.bias_grad_group = p.r ? fb_suggest_bias_grad_group(&p) : 0;
+        if (factor_grads) {
             const int64_t rows = ((int64_t)p.B + group - 1) / group;
             dqb_full = torch::empty({rows, p.Lq, p.H, p.r}, q.options());
             dkb_full = torch::empty({rows, p.Lk, p.H, p.r}, q.options());
@@ -176,7 +179,7 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
             const c10::hip::HIPGuardMasqueradingAsCUDA guard(q.device()); // (torch on ROCm presents its devices as "cuda")
             const hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(q.device().index()).stream();
             check(fb_bwd(&p, stream));
-            if (p.r) {
+            if (factor_grads) {
                 dqb = reduce_like(dqb_full, qb, stream);
                 dkb = reduce_like(dkb_full, kb, stream);
             }

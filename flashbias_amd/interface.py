@@ -227,7 +227,10 @@ def _forward_with_block(q, k, v, q_bias, k_bias, mask, causal, softmax_scale, fa
     return o, lse, p.scale, (p, keep)
 
 
-def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale, factors=None, block=None):
+def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, softmax_scale, factors=None, block=None,
+                         factor_grads=True):
+    """factor_grads=False: neither factor asks for its gradient (constant factors: ALiBi slopes, tables loaded from
+    a file, coordinates); the library is then given no dq_bias / dk_bias and its kernels skip them."""
     lib = _lib.load()
     do = _last_dim_contiguous(do)
     if block is not None and (block[0].q.ptr, block[0].k.ptr, block[0].v.ptr) == (q.data_ptr(), k.data_ptr(), v.data_ptr()):
@@ -240,10 +243,11 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     p.o, p.lse, p.dout = _tensor(o), lse.data_ptr(), _tensor(do)
     p.dq, p.dk, p.dv = _tensor(dq), _tensor(dk), _tensor(dv)
     dqb_full = dkb_full = None
-    if p.r:  # (also when only a folded vector mask makes up the factors)
-        # factors shared by a large batch of short sequences: the kernels sum the gradients of `group` batch
-        # entries themselves and the full-shape tensors shrink by that factor
-        group = p.bias_grad_group = lib.fb_suggest_bias_grad_group(p)
+    p.dq_bias = p.dk_bias = _lib.FbTensor()  # (the block may be the forward's, or an earlier backward's)
+    # factors shared by a large batch of short sequences: a workgroup walks `group` batch entries (it then loads the
+    # factor operand it keeps once), sums their factor gradients itself, and the full-shape tensors shrink by that factor
+    group = p.bias_grad_group = lib.fb_suggest_bias_grad_group(p) if p.r else 0
+    if p.r and factor_grads and q_bias is not None:
         rows = -(-p.B // group)
         dqb_full = torch.empty((rows, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
         dkb_full = torch.empty((rows, p.Lk, p.H, p.r), device=q.device, dtype=q.dtype)
@@ -254,7 +258,7 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     _launch(lib.fb_bwd, p, q.device)
     del keep
     dq_bias = dk_bias = None
-    if q_bias is not None:
+    if dqb_full is not None:
         dq_bias = _reduce_like(dqb_full, q_bias)
         dk_bias = _reduce_like(dkb_full, k_bias)
     return dq, dk, dv, dq_bias, dk_bias
@@ -313,7 +317,8 @@ class FlashBiasFunc(torch.autograd.Function):
         q, k, v, o, q_bias, k_bias, lse, mask = ctx.saved_tensors
         assert not ctx.needs_input_grad[5], "FlashBias does not support mask gradient yet"
         dq, dk, dv, dq_bias, dk_bias = _flash_bias_backward(
-            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale, ctx.kernel_factors, ctx.block)
+            do, q, k, v, o, q_bias, k_bias, lse, mask, ctx.causal, ctx.softmax_scale, ctx.kernel_factors, ctx.block,
+            factor_grads=ctx.needs_input_grad[3] or ctx.needs_input_grad[4])
         return dq, dk, dv, dq_bias, dk_bias, None, None, None
 
 

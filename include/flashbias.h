@@ -85,7 +85,10 @@ typedef struct fb_params {
     fb_tensor dout;             /* bwd in: upstream gradient of o */
     fb_tensor dq, dk, dv;       /* bwd out */
     fb_tensor dq_bias, dk_bias; /* bwd out, full (B, L, H, r) shape: the caller reduces over
-                                   broadcast dims (but see bias_grad_group) */
+                                   broadcast dims (but see bias_grad_group).  Both pointers NULL: the
+                                   factor gradients are not wanted (constant factors) and are neither
+                                   stored nor, in the streamlined kernels, computed; the reference
+                                   always computes them (flash_bias_triton.py:718-719, :725-817) */
     float *delta;               /* backward scratch of fb_bwd_workspace_bytes() bytes, 16-byte aligned, written by the
                                    backward: -delta and lse * log2(e) per query row, as fp32 and as 16-bit parts */
     int32_t bias_grad_group;    /* 0 or 1: as above.  g > 1, for factors that the batch shares (stride_b = 0, the

@@ -112,6 +112,17 @@ def test_check_rejects_backward(mutate, code):
         assert fn(p, None) == code
 
 
+def test_factor_gradients_may_be_left_out():
+    """Both of dq_bias and dk_bias null: the caller does not want them; one of them null: an error."""
+    lib = _lib.load()
+    p = _good(1)
+    p.dq_bias.ptr = p.dk_bias.ptr = None
+    assert lib.fb_check(p, 1) == 0
+    p = _good(1)
+    p.dk_bias.ptr = None
+    assert lib.fb_check(p, 1) == -1
+
+
 def test_grouped_factor_gradients_checks_and_suggestion():
     """bias_grad_group = g: the factor gradients have ceil(B / g) batch rows, so a single group may
     use a zero batch stride; the library suggests groups only for factors shared by a large batch of

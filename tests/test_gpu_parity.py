@@ -594,6 +594,61 @@ def test_large_grids_ragged(gpu_device, B, H, Lq, Lk, r, causal):
     _case(gpu_device, B, Lq, Lk, H, 32, r, torch.bfloat16, causal, seed=13)
 
 
+@pytest.mark.parametrize("B,H,Lq,Lk,d,r,causal,dtype", [
+    (2, 4, 1024, 1024, 32, 8, False, torch.bfloat16),    # streamlined kernels, one mixed backward launch
+    (8, 16, 1000, 1000, 32, 8, True, torch.float16),     # streamlined dq and dk/dv kernels on a grid that fills the chip
+    (1, 8, 2048, 2048, 32, 5, False, torch.bfloat16),    # rank 5 with small entries: padded to 8, streamlined
+    (3, 4, 300, 520, 32, 16, False, torch.bfloat16),     # general kernels
+    (2, 2, 200, 333, 64, 32, True, torch.bfloat16),
+    (40, 16, 256, 256, 32, 16, False, torch.bfloat16),   # factors shared by a large batch (groups of batch entries)
+])
+def test_constant_factors_skip_their_gradients(gpu_device, B, H, Lq, Lk, d, r, causal, dtype):
+    """Factors that do not require a gradient (ALiBi slopes, tables loaded from a file, coordinates): the library
+    is given no dq_bias / dk_bias; o, dq, dk, dv are bit for bit those of the call that computes all five."""
+    shared = B >= 32
+    q, k, v, qb, kb, do = make_inputs(B, Lq, Lk, H, d, r, dtype, seed=77, bq=(shared, False), bk=(shared, False))
+    dev = gpu_device
+
+    def run(factor_grads):
+        leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
+        fac = [t.to(dev).requires_grad_(factor_grads) for t in (qb, kb)]
+        o = flash_bias_func(leaves[0], leaves[1], leaves[2], fac[0], fac[1], None, causal, None)
+        grads = torch.autograd.grad(o, leaves + (fac if factor_grads else []), do.to(dev))
+        return [o.detach()] + list(grads)
+
+    full, part = run(True), run(False)
+    assert len(full) == 6 and len(part) == 4
+    for name, a, b in zip(("o", "dq", "dk", "dv"), full, part):
+        assert torch.equal(a, b), name
+    # and through the C ABI: null outputs are accepted, one of two is not
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _params, _stream, _tensor
+    lib = _lib.load()
+    qd, kd, vd, qbd, kbd, dod = [t.to(dev) for t in (q, k, v, qb, kb, do)]
+    p, keep = _params(qd, kd, vd, qbd, kbd, None, causal, None)
+    o = torch.empty_like(qd)
+    lse = torch.empty((B, H, Lq), device=dev, dtype=torch.float32)
+    p.o, p.lse = _tensor(o), lse.data_ptr()
+    _lib.check_status(lib.fb_fwd(p, _stream()))
+    outs = [torch.empty_like(t) for t in (qd, kd, vd)]
+    p.dout, p.dq, p.dk, p.dv = _tensor(dod), _tensor(outs[0]), _tensor(outs[1]), _tensor(outs[2])
+    scratch = torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=dev, dtype=torch.float32)
+    p.delta = scratch.data_ptr()
+    for name in ("fb_bwd", "fb_bwd_static"):
+        for t in outs:
+            t.zero_()
+        _lib.check_status(getattr(lib, name)(p, _stream()))
+        torch.cuda.synchronize()
+        for nm, a, b in zip(("dq", "dk", "dv"), full[1:4], outs):
+            assert torch.equal(a, b), (name, nm)
+    _lib.check_status(lib.fb_bwd_preprocess(p, _stream()))
+    _lib.check_status(lib.fb_bwd_dkv(p, _stream()))
+    _lib.check_status(lib.fb_bwd_dq(p, _stream()))
+    torch.cuda.synchronize()
+    for nm, a, b in zip(("dq", "dk", "dv"), full[1:4], outs):
+        assert torch.equal(a, b), ("phases", nm)
+
+
 def _random_configurations(n, seed):
     """n configurations drawn with a fixed seed from everything the operator accepts: head dims 8 ... 128
     (not only multiples of 8), ranks 0 ... 64, lengths 1 ... 900 on either side, either element type,
