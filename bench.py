@@ -165,6 +165,22 @@ def _autograd_ms(leaves, extra, do, steps, warmup, prepare=None):
     return t_fwd, _time_events(fb, steps, warmup)
 
 
+def _constant_factors_ms(leaves, extra, do, steps, warmup):
+    """fwd+bwd milliseconds of the same step when the factors are constants (no gradient asked of them,
+    as in the reference's own applications: ALiBi slopes, attention_with_alibi_bias.py:44-52; tables
+    loaded from a file, swin_transformer_v2.py:147-152): the operator then computes dq, dk, dv only."""
+    import torch
+    from flashbias_amd import flash_bias_func
+    mask, causal, scale = extra
+    fac = [t.detach() for t in leaves[3:5]]
+
+    def fb():
+        o = flash_bias_func(leaves[0], leaves[1], leaves[2], fac[0], fac[1], mask, causal, scale)
+        return torch.autograd.grad(o, leaves[:3], do)
+
+    return _time_events(fb, steps, warmup)
+
+
 def _graph_ms(leaves, extra, do, steps, warmup):
     """fwd+bwd milliseconds of the same autograd step captured once in a HIP graph and replayed: what
     a training loop that captures its step pays, without the host's per-call work (which bounds the
@@ -258,6 +274,7 @@ def _sweep(dev, steps, warmup, only=None):
         leaves = [t.requires_grad_(True) for t in (q, k, v, qb, kb)]
         t_fwd, t_fb = _autograd_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
         t_graph = _graph_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
+        t_const = _constant_factors_ms(leaves, (None, causal, 1.0 / math.sqrt(d)), do, steps, warmup)
         f_fwd, f_bwd = workloads.flops(B, H, L, L, d, r, causal)
         # algorithmic HBM bytes of a step: every input read once per pass, every output written once
         # (forward: q k v factors -> o, lse; backward: q k v o dO factors lse -> dq dk dv and the factor
@@ -271,6 +288,8 @@ def _sweep(dev, steps, warmup, only=None):
                     "fwd_bwd_graph_ms": None if t_graph is None else round(t_graph, 4),
                     "graph_pct_of_bf16_mfma_peak": None if t_graph is None else
                     round(100 * (f_fwd + f_bwd) / t_graph / 1e9 / PEAK_BF16_TFLOPS, 2),
+                    # (not comparable with fwd_bwd_ms: two of the five gradients are not computed)
+                    "fwd_bwd_ms_constant_factors": round(t_const, 4),
                     "hbm_algorithmic_gb": round(hbm / 1e9, 3), "hbm_gbs": round(hbm / t_fb / 1e6, 1),
                     "pct_of_hbm_peak": round(100 * hbm / t_fb / 1e6 / PEAK_HBM_GBS, 2)})
         del q, k, v, qb, kb, do, leaves

@@ -32,7 +32,9 @@ namespace fb {
 // its LDS stages small enough for two waves per SIMD, which is worth recomputing S.
 // FOLD_: the scores are scale * (q k^T + q_b (k_b / scale)^T), no multiply per score for the scale
 // (the launcher says when that is exact).
-template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, int PART_ = 0, bool FOLD_ = false>
+// BG_: also accumulate dk_bias (false: the caller does not want the factor gradients; the accumulator blocks that
+// hold nothing but dk_bias are then left out).
+template <class T, int NKD_, int NKR_, int NDV_, bool VEC_, bool MASK_, int PART_ = 0, bool FOLD_ = false, bool BG_ = true>
 struct DkvCfg {
     static constexpr bool FOLD = FOLD_;
     static_assert(!FOLD_ || (VEC_ && !MASK_), "folded scale: direct loader, no additive mask");
@@ -46,7 +48,9 @@ struct DkvCfg {
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dK | dK_b]^T
     // ... of which this instantiation accumulates [MB0, MB1)
-    static constexpr int MB0 = PART_ == 4 ? MB / 2 : 0, MB1 = PART_ == 1 ? 0 : PART_ == 3 ? MB / 2 : MB;
+    static constexpr int MB0 = PART_ == 4 ? MB / 2 : 0,
+                         MB1 = PART_ == 1 ? 0 : PART_ == 3 ? MB / 2 : (BG_ ? MB : (NKD_ + 1) / 2);
+    static_assert(BG_ || PART_ == 0, "");
     static constexpr int KBW = 1; // key blocks per wave
     static constexpr int BN = 32 * KBW * NWAVES;              // keys per workgroup
     static constexpr int QBLK = PART_ == 0 ? 2 : 1, BMQ = 32 * QBLK; // queries per step
@@ -601,9 +605,9 @@ bwd_dkv_kernel(const BwdArgs a) {
     bwd_dkv_body<T, C>(a, blockIdx.x);
 }
 
-template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART, bool FOLD>
+template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, int PART, bool FOLD, bool BG = true>
 static hipError_t launch_dkv_part(const BwdArgs &a0, hipStream_t stream) {
-    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK, PART, FOLD> C;
+    typedef DkvCfg<T, NKD, NKR, NDV, VEC, MASK, PART, FOLD, BG> C;
     BwdArgs a = a0;
     a.ntiles_n = (a.Lk + C::BN - 1) / C::BN;
     auto kern = bwd_dkv_kernel<T, C>;
@@ -633,6 +637,10 @@ static hipError_t launch_dkv_vec(const BwdArgs &a, hipStream_t stream) {
         }
         return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 4, FOLD>(a, stream);
     } else {
+        // head dim 32, aligned, unmasked, no dk_bias wanted: the instantiation without its products
+        if constexpr (NKD == 2 && NKR > 0 && NKR <= 2 && VEC && !MASK) {
+            if (!a.dkb.ptr) return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 0, FOLD, false>(a, stream);
+        }
         return launch_dkv_part<T, NKD, NKR, NDV, VEC, MASK, 0, FOLD>(a, stream);
     }
 }

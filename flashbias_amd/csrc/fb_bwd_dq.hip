@@ -25,7 +25,10 @@ namespace fb {
 // FOLD_: the scores are scale * (q k^T + (q_b / scale) k_b^T), one MFMA chain and no FMA per
 // score for the scale (the launcher says when that is exact).
 // KB1_: 32-key tiles (half the LDS per stage: two workgroups per CU at head dims above 64).
-template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_, bool QB2_ = true, bool FOLD_ = false, bool KB1_ = false>
+// BG_: also accumulate dq_bias (false: the caller does not want the factor gradients; the accumulator blocks that
+// hold nothing but dq_bias are then left out of the products).
+template <class T, int NKD_, int NKR_, bool VEC_, bool MASK_, bool QB2_ = true, bool FOLD_ = false, bool KB1_ = false,
+          bool BG_ = true>
 struct DqCfg {
     static constexpr bool FOLD = FOLD_;
     static_assert(!FOLD_ || (VEC_ && !MASK_), "folded scale: direct loader, no additive mask");
@@ -37,6 +40,7 @@ struct DqCfg {
     static constexpr int NWAVES = 4, NTHREADS = 64 * NWAVES;
     static constexpr int NK = NKD + NKR;
     static constexpr int MB = (NK + 1) / 2; // 32-row blocks of [dQ | dQ_b]^T
+    static constexpr int MBE = BG_ ? MB : (NKD + 1) / 2; // ... of which the key loop accumulates the first MBE
     static constexpr int QBLK = (QB2_ && NK <= 3 && !MASK_) ? 2 : 1; // the mask values need the registers of the second block
     static constexpr int BM = NWAVES * QBLK * 32;
     static constexpr int KBLK = KB1_ ? 1 : 2, BN = 32 * KBLK;
@@ -487,7 +491,7 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int n = 0; n < C::MB; ++n) {
+                    for (int n = 0; n < C::MBE; ++n) {
                         const u32x4_t kt = lds_read_a_tr<C::ROWCH>(sK, kb * 32 + 16 * t, 32 * n, c, g);
 #pragma unroll
                         for (int qb = 0; qb < C::QBLK; ++qb) acc[qb][n] = T::mfma(kt, dsp[qb][t], acc[qb][n]);
@@ -529,9 +533,9 @@ bwd_dq_kernel(const BwdArgs a) {
     bwd_dq_body<T, C>(a, blockIdx.x);
 }
 
-template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2, bool FOLD, bool KB1 = false>
-static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
-    typedef DqCfg<T, NKD, NKR, VEC, MASK, QB2, FOLD, KB1> C;
+template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2, bool FOLD, bool KB1, bool BG>
+static hipError_t launch_dq_qb_bg(const BwdArgs &a0, hipStream_t stream) {
+    typedef DqCfg<T, NKD, NKR, VEC, MASK, QB2, FOLD, KB1, BG> C;
     BwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = bwd_dq_kernel<T, C>;
@@ -542,6 +546,15 @@ static hipError_t launch_dq_qb(const BwdArgs &a0, hipStream_t stream) {
     const int64_t total = (int64_t)a.ntiles_m * ((a.B + group - 1) / group) * a.H;
     a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, once);
     return launch_flat(kern, total, C::NTHREADS, C::LDS_BYTES, stream, a);
+}
+
+template <class T, int NKD, int NKR, bool VEC, bool MASK, bool QB2, bool FOLD, bool KB1 = false>
+static hipError_t launch_dq_qb(const BwdArgs &a, hipStream_t stream) {
+    // head dim 32, aligned, unmasked, no dq_bias wanted: the instantiation without its products
+    if constexpr (NKD == 2 && NKR > 0 && NKR <= 2 && VEC && !MASK && !KB1) {
+        if (!a.dqb.ptr) return launch_dq_qb_bg<T, NKD, NKR, VEC, MASK, QB2, FOLD, KB1, false>(a, stream);
+    }
+    return launch_dq_qb_bg<T, NKD, NKR, VEC, MASK, QB2, FOLD, KB1, true>(a, stream);
 }
 
 // 256-query workgroups (two blocks per wave) once every compute unit has two of them (four under
