@@ -13,7 +13,7 @@ FB_F16, FB_BF16, FB_F32 = 0, 1, 2
 FB_MASK_NONE, FB_MASK_VECTOR, FB_MASK_MATRIX = 0, 1, 2
 
 #: every symbol that include/flashbias.h declares
-EXPORTS = ("fb_version", "fb_last_error", "fb_bwd_workspace_bytes", "fb_suggest_bias_grad_group", "fb_check", "fb_fwd", "fb_bwd",
+EXPORTS = ("fb_version", "fb_init", "fb_last_error", "fb_bwd_workspace_bytes", "fb_suggest_bias_grad_group", "fb_check", "fb_fwd", "fb_bwd",
            "fb_sum_over_batch",
            "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static")
 
@@ -59,6 +59,7 @@ def load():
         if not hasattr(lib, name):
             raise ImportError(f"{LIB_PATH} does not export {name}")
     lib.fb_version.restype = ctypes.c_int
+    lib.fb_init.restype = ctypes.c_int
     lib.fb_last_error.restype = ctypes.c_char_p
     lib.fb_bwd_workspace_bytes.argtypes = [ctypes.POINTER(FbParams)]
     lib.fb_bwd_workspace_bytes.restype = ctypes.c_size_t

@@ -171,6 +171,13 @@ int launched(hipError_t e, const char *what) {
 
 extern "C" {
 
+int fb_init(void) {
+    fb::api_clear_error();
+    hipError_t e = hipSuccess;
+    if (!static_scratch(&e)) return launched(e, "fb_init (hipGetSymbolAddress)");
+    return FB_OK;
+}
+
 int fb_fwd(const fb_params *p, void *stream) {
     const int rc = fb_check(p, 0);
     if (rc) return rc;

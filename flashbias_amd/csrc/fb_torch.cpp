@@ -122,10 +122,7 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
             qb = channel_contiguous(*qb_in);
             kb = channel_contiguous(*kb_in);
         }
-        if (mask_in.has_value() && mask_in->defined()) {
-            TORCH_CHECK(!mask_in->requires_grad(), "FlashBias does not support mask gradient yet");
-            mask = channel_contiguous(*mask_in);
-        }
+        if (mask_in.has_value() && mask_in->defined()) mask = channel_contiguous(*mask_in);
         const double scale = softmax_scale != 0.0 ? softmax_scale : 1.0 / std::sqrt((double)q.size(3));
         tensor_list keep;
         fb_params p = block(q, k, v, qb, kb, mask, causal, scale, keep);
@@ -144,6 +141,8 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
     }
 
     static tensor_list backward(AutogradContext *ctx, tensor_list grads) {
+        // (as the reference: only a backward that is asked for the mask's gradient fails, flash_bias_triton.py:1391)
+        TORCH_CHECK(!ctx->needs_input_grad(5), "FlashBias does not support mask gradient yet");
         const auto saved = ctx->get_saved_variables();
         const Tensor &q = saved[0], &k = saved[1], &v = saved[2], &o = saved[3], &lse = saved[4];
         const Tensor &qb = saved[5], &kb = saved[6], &mask = saved[7];
@@ -163,7 +162,10 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
         // factors shared by a large batch of short sequences: a workgroup walks `group` batch entries (it then loads
         // the factor operand it keeps once), sums their factor gradients itself, and the full-shape tensors shrink by
         // that factor
-        const int group = p.bias_grad_group = p.r ? fb_suggest_bias_grad_group(&p) : 0;
+        // (only for factors saved with a batch of one: a factor expanded over the batch by its caller also has batch
+        // stride 0, but autograd wants its gradient in the expanded shape)
+        const bool shared = p.r && qb.size(0) == 1 && kb.size(0) == 1 && p.B > 1;
+        const int group = p.bias_grad_group = p.r ? (shared ? fb_suggest_bias_grad_group(&p) : 1) : 0;
         if (factor_grads) {
             const int64_t rows = ((int64_t)p.B + group - 1) / group;
             dqb_full = torch::empty({rows, p.Lq, p.H, p.r}, q.options());
@@ -197,6 +199,8 @@ Tensor flash_bias(const Tensor &q, const Tensor &k, const Tensor &v, const c10::
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "flash_bias_func with its autograd function in C++ (kernel-ready inputs; see flashbias_amd/interface.py)";
+    // what this module was compiled against: the caller compares both with the library it loaded
+    m.def("abi", []() { return std::make_pair((int)FB_VERSION, (int)sizeof(fb_params)); });
     m.def("flash_bias", &flash_bias, py::arg("q"), py::arg("k"), py::arg("v"), py::arg("q_bias") = py::none(),
           py::arg("k_bias") = py::none(), py::arg("mask") = py::none(), py::arg("causal") = false,
           py::arg("softmax_scale") = 0.0);

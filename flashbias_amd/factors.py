@@ -69,6 +69,23 @@ def distance_factors(x_q, x_k, alpha, dtype=torch.float32):
     return q_bias[:, :, None, :].to(dtype), k_bias[:, :, None, :].to(dtype)
 
 
+def pad_rank(q_bias, k_bias, multiple=8):
+    """The factors with zero columns appended up to the next multiple of ``multiple`` (the product
+    q_bias k_bias^T is unchanged).  ``flash_bias_func`` pads ranks that are not multiples of 8 by
+    itself on every call, and ranks below 8 to 16, because the rank-8 kernels fold the softmax scale
+    into a 16-bit operand and carry each bias term q_bias[i, c] k_bias[j, c] with a relative error of
+    2^-17: harmless for terms up to a few hundred (0.002 in the logits at 256), not for ALiBi's
+    closed form (terms in the thousands).  Constant factors with small terms (the distance bias over
+    points in a unit box: at most 2 alpha) are padded to 8 here, once, by the caller who knows them;
+    the operator then runs the rank-8 kernels and pads nothing per call."""
+    rank = q_bias.shape[-1]
+    assert k_bias.shape[-1] == rank
+    pad = (-rank) % multiple
+    if pad == 0:
+        return q_bias, k_bias
+    return torch.nn.functional.pad(q_bias, (0, pad)), torch.nn.functional.pad(k_bias, (0, pad))
+
+
 def svd_factors(bias, rank, dtype=torch.float32):
     """Best rank-``rank`` factors (Eckart-Young) of a per-head bias table (H, Lq, Lk).
     Returns q_bias (1, Lq, H, rank), k_bias (1, Lk, H, rank) and the relative Frobenius error

@@ -12,7 +12,6 @@ stream.  Differences from the reference, all on purpose:
 * ``softmax_scale`` of ``None`` or 0 gives ``1/sqrt(d)`` as in the reference (:1110).
 """
 import math
-import weakref
 
 import torch
 
@@ -71,38 +70,6 @@ def _fold_vector_mask(q, q_bias, k_bias, mask):
     return q_new, k_new
 
 
-#: bound on sum_c max_i |q_bias[i, c]| max_j |k_bias[j, c]| (an upper bound of every |bias_ij|) below which
-#: factors of rank < 8 are padded to rank 8: the kernels for rank 8 carry a bias term with a relative error of
-#: 2^-17, 0.002 in the logits at this bound.
-_SMALL_BIAS_BOUND = 256.0
-_bias_bound_cache = {}  # id(q_bias) -> (weakref(q_bias), weakref(k_bias), versions, bound)
-
-
-def _bias_terms_are_small(q_bias, k_bias):
-    """Whether the factors' entries are small enough for the rank-8 kernels (see _SMALL_BIAS_BOUND).
-    Decided on the host from two reductions on the device, i.e. with a synchronisation, so only for
-    leaf tensors (buffers, parameters, constants such as the geometry factors of a PDE solver: the
-    same objects call after call) and cached per tensor pair and version; while a graph is being
-    captured only the cache is consulted.  Everything else gets the conservative answer."""
-    if not (q_bias.is_leaf and k_bias.is_leaf):
-        return False
-    key = id(q_bias)
-    versions = (q_bias._version, k_bias._version)
-    hit = _bias_bound_cache.get(key)
-    if hit is not None and hit[0]() is q_bias and hit[1]() is k_bias and hit[2] == versions:
-        return hit[3] <= _SMALL_BIAS_BOUND
-    if torch.cuda.is_current_stream_capturing():
-        return False  # (a pair seen before the capture keeps its answer: that needs no synchronisation)
-    with torch.no_grad():
-        rank = q_bias.shape[-1]
-        bound = float((q_bias.detach().float().abs().reshape(-1, rank).amax(0)
-                       * k_bias.detach().float().abs().reshape(-1, rank).amax(0)).sum())
-    if len(_bias_bound_cache) > 64:
-        _bias_bound_cache.clear()
-    _bias_bound_cache[key] = (weakref.ref(q_bias), weakref.ref(k_bias), versions, bound)
-    return bound <= _SMALL_BIAS_BOUND
-
-
 def _prepare_factors(q, k, q_bias, k_bias, mask):
     """What the kernels get in place of (q_bias, k_bias, mask): a large vector mask folded into the
     factors, the rank zero-padded to a multiple of 8, the channel dimension contiguous.  Done once
@@ -128,9 +95,10 @@ def _prepare_factors(q, k, q_bias, k_bias, mask):
             # and a rank of 16 selects the kernels that keep the factors as they are and apply the
             # softmax scale to the fp32 accumulator.  The kernels that fold the scale into a 16-bit
             # operand (rank 8) carry every bias term with a relative error of 2^-17, which is 0.05 in
-            # the logits at |term| = 7000.  Constant factors with small entries (a distance bias over
-            # points in a unit box) do take rank 8.
-            target = 8 if rank < 8 and _bias_terms_are_small(q_bias, k_bias) else (16 if rank < 8 else -(-rank // 8) * 8)
+            # the logits at |term| = 7000.  A caller whose factors have small entries (a distance bias
+            # over points in a unit box) opts in to rank 8 by padding them itself, once
+            # (factors.pad_rank): the choice depends on nothing but the shapes it passes.
+            target = 16 if rank < 8 else -(-rank // 8) * 8
             pad = (0, target - rank)
             q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
         # (padding a permuted view keeps its permuted layout)
@@ -246,7 +214,10 @@ def _flash_bias_backward(do, q, k, v, o, q_bias, k_bias, lse, mask, causal, soft
     p.dq_bias = p.dk_bias = _lib.FbTensor()  # (the block may be the forward's, or an earlier backward's)
     # factors shared by a large batch of short sequences: a workgroup walks `group` batch entries (it then loads the
     # factor operand it keeps once), sums their factor gradients itself, and the full-shape tensors shrink by that factor
-    group = p.bias_grad_group = lib.fb_suggest_bias_grad_group(p) if p.r else 0
+    # (only for factors that are saved with a batch of one: a factor expanded over the batch by its caller also has
+    # batch stride 0, but autograd wants its gradient in the expanded shape)
+    shared = q_bias is not None and q_bias.shape[0] == 1 and k_bias.shape[0] == 1 and p.B > 1
+    group = p.bias_grad_group = (lib.fb_suggest_bias_grad_group(p) if shared else 1) if p.r else 0
     if p.r and factor_grads and q_bias is not None:
         rows = -(-p.B // group)
         dqb_full = torch.empty((rows, p.Lq, p.H, p.r), device=q.device, dtype=q.dtype)
@@ -332,8 +303,12 @@ def _extension():
     if _ext is False:
         try:
             from . import _fb_torch
-            _lib.load()
-            _ext = _fb_torch
+            lib = _lib.load()
+            # (a module built against another version of the parameter block would fail every call with
+            # FB_ERR_ABI: the Python function serves instead)
+            import ctypes
+            ok = getattr(_fb_torch, "abi", lambda: None)() == (lib.fb_version(), ctypes.sizeof(_lib.FbParams))
+            _ext = _fb_torch if ok else None
         except ImportError:
             _ext = None
     return _ext

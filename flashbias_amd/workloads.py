@@ -84,13 +84,17 @@ def swin(windows=4096, window=16, H=16, d=32, r=16, dtype=torch.bfloat16, seed=0
     return w
 
 
-def pde(N=32768, H=8, d=32, alpha=10.0, dtype=torch.bfloat16, seed=0):
-    """Spatial-distance bias -alpha |x_i - x_j|^2 over N points in [0,1]^3, exact rank 5."""
+def pde(N=32768, H=8, d=32, alpha=10.0, dtype=torch.bfloat16, seed=0, pad_to=8):
+    """Spatial-distance bias -alpha |x_i - x_j|^2 over N points in [0,1]^3, exact rank 5.  The factors'
+    terms are at most 2 alpha in magnitude, so they are stored with three zero columns (rank 8,
+    factors.pad_rank), which selects the rank-8 kernels; pad_to=None leaves them at rank 5."""
     g = torch.Generator().manual_seed(seed)
     q, k, v, do = _qkv(1, N, N, H, d, g, dtype)
     x = torch.rand(1, N, 3, generator=g)
     qb, kb = factors.distance_factors(x, x, alpha, dtype)
-    return _pack(q, k, v, do, qb, kb, False, 1.0 / math.sqrt(d), points=x)
+    if pad_to:
+        qb, kb = factors.pad_rank(qb, kb, pad_to)
+    return _pack(q, k, v, do, qb, kb, False, 1.0 / math.sqrt(d), points=x, rank=5)
 
 
 def pairformer(N=768, H=4, d=32, r=32, dtype=torch.bfloat16, seed=0):

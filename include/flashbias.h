@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define FB_VERSION 2
+#define FB_VERSION 3
 #define FB_MAX_HEADDIM 128 /* flash_bias_triton.py:1106 */
 #define FB_MAX_RANK 128
 /* Size of the library-owned scratch buffer used by fb_bwd_static (one copy per GPU, held until the
@@ -103,6 +103,14 @@ typedef struct fb_params {
 /* Library / ABI version. */
 int fb_version(void);
 
+/* Optional set-up for the current device: looks up the address of the static scratch array that
+ * fb_bwd_static uses (one hipGetSymbolAddress per device, cached), so that no later call has to.
+ * fb_bwd_static does the same on its first call on a device; a caller that wants that first call
+ * inside a HIP graph capture calls fb_init() (or fb_bwd_static once, eagerly) on the device
+ * beforehand, because a symbol lookup is not a stream operation and must not happen while a
+ * stream is capturing.  Launches nothing, allocates nothing.  No counterpart in the reference. */
+int fb_init(void);
+
 /* Text of the last error on this thread ("" if none). */
 const char *fb_last_error(void);
 
@@ -149,7 +157,9 @@ int fb_bwd(const fb_params *p, void *stream);
  * anything it calls allocates or frees memory.  Returns FB_ERR_SHAPE when
  * fb_bwd_workspace_bytes(p) exceeds FB_STATIC_SCRATCH_BYTES.  All calls on one GPU share that
  * GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls
- * ordered on one stream are safe.  Nothing in the array has to be cleared between calls. */
+ * ordered on one stream are safe.  Nothing in the array has to be cleared between calls.  The
+ * first call on a device looks the array's address up (see fb_init): make it, or fb_init(), outside
+ * graph capture. */
 int fb_bwd_static(const fb_params *p, void *stream);
 
 /* The last step of the backward for factors that every batch entry shares: the kernels write such

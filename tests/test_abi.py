@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.fb_version() == 2
+    assert lib.fb_version() == 3
 
 
 def test_workspace_size_query():

@@ -95,8 +95,11 @@ def test_workloads_are_seeded_and_shaped():
     assert w["causal"] and w["q_bias"].shape == (1, 128, 6, 2)
     w = workloads.swin(windows=3, window=4, H=2, r=4)
     assert w["q"].shape == (3, 16, 2, 32) and w["q_bias"].shape == (1, 16, 2, 4)
-    w = workloads.pde(N=64, H=2)
-    assert w["q_bias"].shape == (1, 64, 1, 5)
+    w = workloads.pde(N=64, H=2)  # rank 5, stored with three zero columns
+    assert w["q_bias"].shape == (1, 64, 1, 8) and not w["q_bias"][..., 5:].any() and not w["k_bias"][..., 5:].any()
+    w5 = workloads.pde(N=64, H=2, pad_to=None)
+    assert w5["q_bias"].shape == (1, 64, 1, 5) and torch.equal(w5["q_bias"], w["q_bias"][..., :5])
+    assert factors.pad_rank(w["q_bias"], w["k_bias"], 8)[0] is w["q_bias"]
     w = workloads.pairformer(N=16, H=2, r=8)
     assert w["q"].shape == (16, 16, 2, 32) and w["k_bias"].shape == (1, 16, 2, 8)
 
