@@ -141,11 +141,13 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
     }
 
     static tensor_list backward(AutogradContext *ctx, tensor_list grads) {
-        // (as the reference: only a backward that is asked for the mask's gradient fails, flash_bias_triton.py:1391)
-        TORCH_CHECK(!ctx->needs_input_grad(5), "FlashBias does not support mask gradient yet");
         const auto saved = ctx->get_saved_variables();
         const Tensor &q = saved[0], &k = saved[1], &v = saved[2], &o = saved[3], &lse = saved[4];
         const Tensor &qb = saved[5], &kb = saved[6], &mask = saved[7];
+        // as the reference, only a backward that is asked for the mask's gradient fails (flash_bias_triton.py:1371).
+        // (The graph edges count the tensor arguments that were given: q, k, v, then the factors, then the mask.)
+        if (mask.defined())
+            TORCH_CHECK(!ctx->needs_input_grad(qb.defined() ? 5 : 3), "FlashBias does not support mask gradient yet");
         const bool causal = ctx->saved_data["causal"].toBool();
         const double scale = ctx->saved_data["scale"].toDouble();
         const Tensor dout = channel_contiguous(grads[0]);

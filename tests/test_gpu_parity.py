@@ -383,11 +383,15 @@ def test_mask_gradient_is_refused_in_backward_only(gpu_device):
     q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(1, 64, 64, 2, 32, 8, dt, seed=3)]
     mask = torch.zeros(1, 2, 64, 64, device=dev, dtype=dt, requires_grad=True)
     for fn in (flash_bias_func, FlashBiasFunc.apply):
-        with torch.no_grad():
-            want = fn(q, k, v, qb, kb, mask.detach(), False, None)
-            assert torch.equal(fn(q, k, v, qb, kb, mask, False, None), want)
-        o = fn(q.clone().requires_grad_(True), k, v, qb, kb, mask, False, None)
-        with pytest.raises((AssertionError, RuntimeError), match="mask gradient"):
+        for fa, fb_ in ((qb, kb), (None, None)):
+            with torch.no_grad():
+                want = fn(q, k, v, fa, fb_, mask.detach(), False, None)
+                assert torch.equal(fn(q, k, v, fa, fb_, mask, False, None), want)
+            o = fn(q.clone().requires_grad_(True), k, v, fa, fb_, mask, False, None)
+            with pytest.raises((AssertionError, RuntimeError), match="mask gradient"):
+                o.backward(do)
+            # a mask that asks for nothing: the backward runs
+            o = fn(q.clone().requires_grad_(True), k, v, fa, fb_, mask.detach(), False, None)
             o.backward(do)
 
 
