@@ -20,6 +20,8 @@ FB_DECL(f16_1) FB_DECL(f16_2) FB_DECL(f16_4) FB_DECL(f16_8)
 #undef FB_DECL
 hipError_t launch_bwd_both_bf16_2(const BwdArgs &a, hipStream_t stream);
 hipError_t launch_bwd_both_f16_2(const BwdArgs &a, hipStream_t stream);
+hipError_t launch_bwd_win_bf16_2(const BwdArgs &a, hipStream_t stream);
+hipError_t launch_bwd_win_f16_2(const BwdArgs &a, hipStream_t stream);
 
 hipError_t launch_fwd(const FwdArgs &a, bool bf16, hipStream_t stream) {
     switch (nkd_of(a.d)) {
@@ -50,6 +52,10 @@ hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream) {
 // dq and dk/dv workgroups of the streamlined kernels in one launch (fb_bwd_both.hip; head dim 32)
 hipError_t launch_bwd_both(const BwdArgs &a, bool bf16, hipStream_t stream) {
     return bf16 ? launch_bwd_both_bf16_2(a, stream) : launch_bwd_both_f16_2(a, stream);
+}
+// all five gradients of a short sequence in one workgroup (fb_bwd_win.hip; head dim 32)
+hipError_t launch_bwd_win(const BwdArgs &a, bool bf16, hipStream_t stream) {
+    return bf16 ? launch_bwd_win_bf16_2(a, stream) : launch_bwd_win_f16_2(a, stream);
 }
 } // namespace fb
 
@@ -244,6 +250,8 @@ int fb_bwd(const fb_params *p, void *stream) {
     const int rc = fb_check(p, 1);
     if (rc) return rc;
     fb::BwdArgs a = bwd_args(p);
+    if (fb::window_backward(a)) // whole sequences of at most 256 positions: one workgroup per (batch, head), one launch
+        return launched(fb::launch_bwd_win(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd (window)");
     if (fb::mixed_backward(a)) {
         // small grids of the streamlined kernels: the preprocess step, then one launch that holds the dq and
         // the dk/dv workgroups side by side (same bits as the two launches)

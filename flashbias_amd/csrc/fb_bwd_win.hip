@@ -1,0 +1,338 @@
+// Backward FlashBias attention for gfx950, window regime: all five gradients of one (batch, head)
+// in one workgroup when the whole sequence fits it (Lq, Lk <= 256: the window attention of
+// 2_Vision_Transformer/swin_transformer_v2.py:178-203).  Replaces the key-block loop of
+// _bwd_kernel_one_col_block (flash_bias/flash_bias_triton.py:575-869) including its dq / dq_bias
+// updates (:725-817), which the reference adds with atomics and the long-sequence kernels of this
+// library (fb_bwd_dkv.hip, fb_bwd_dq.hip) recompute in a second, query-stationary kernel.
+//
+// Sequences this short are bound by memory, not by arithmetic: the two-kernel backward reads q, k,
+// v, o, dO twice and recomputes S and dP.  Here a workgroup of 8 waves holds the window's [Q | Q_b],
+// dO and [K | K_b] in LDS (copied there once, straight from global memory; the query-side tiles of the next
+// window are requested while the current one finishes) and wave w owns keys [32 w, 32 w + 32) with K, K_b, V
+// in registers.  The per-query statistics (delta = rowsum(o * dO), lse * log2 e) are formed by the workgroup
+// itself at the top of a window: no preprocess launch, no scratch buffer.  Per step of 128 queries:
+//
+//   phase 1 (lane = key, as in the dk/dv kernel): S, P = exp(S - lse), dP = dO V^T - delta,
+//           dS = P * dP; dV^T += dO^T P, [dK | dK_b]^T += [Q | Q_b]^T dS with P and dS fed from
+//           registers; dS also goes to LDS as a (256 keys x 128 queries) tile
+//   phase 2 (lane = query): [dQ | dQ_b]^T (64 channels x 128 queries) = [K | K_b]^T dS^T, a small GEMM
+//           over the 256 keys with both operands read column-wise from LDS (transposing reads):
+//           eight 32 x 32 output blocks, one per wave.  The four dq blocks are written at once; the
+//           four dq_bias blocks stay in registers, and since the step's dq_bias blocks go to waves
+//           4 step .. 4 step + 3, every wave ends up holding exactly one of the window's eight.
+//
+// dq needs no sum across workgroups because the workgroup sees every key.  As in the other backward
+// kernels a workgroup walks `group` consecutive batch entries and keeps the factor gradients in
+// registers across them (factors shared by the batch).  All sums have a fixed order: the results
+// are bit-reproducible.
+#define FB_BODIES_ONLY
+#include "fb_bwd_dkv.hip"
+
+namespace fb {
+
+// NKR_: 16-wide steps of the rank (0, 1, 2).  FOLD_: the scores are scale * (q k^T + q_b k_b^T), no multiply per
+// score for the scale (no factors, or a scale of exactly 1).  BG_: also form dq_bias and dk_bias.
+template <class T, int NKR_, bool FOLD_, bool BG_>
+struct WinCfg {
+    static constexpr int NKD = 2, NKR = NKR_, NK = NKD + NKR_, NDV = 1, KBW = 1;
+    static constexpr bool FOLD = FOLD_, BG = BG_ && NKR_ > 0, VEC = true, DO_DV = true, DO_DK = true;
+    static constexpr int NWAVES = 8, NTHREADS = 64 * NWAVES;
+    static constexpr int BN = 32 * NWAVES, LQ = 256, BMQ = 128, QBLK = BMQ / 32;
+    static constexpr int ROWCH = 8;   // 128-byte rows: [Q | Q_b], [K | K_b]
+    static constexpr int ROWCHS = 16; // 256-byte rows: the 128 queries of a key's dS
+    static constexpr int MB = (NK + 1) / 2, MB0 = 0, MB1 = BG ? MB : 1; // 32-row blocks of [dK | dK_b]^T
+    // 16-bit elements; the dO tile is a dense region of 64-byte rows (fb_lean_tiles.h)
+    static constexpr int SQ = LQ * 64, SDO = LQ * 32, SK = BN * 64, SDS = BN * 128;
+    static constexpr int STAT_FLOATS = 2 * LQ;
+    static constexpr int LDS_BYTES = 2 * (SQ + SDO + SK + SDS) + 4 * STAT_FLOATS;
+    static_assert(LDS_BYTES <= 160 * 1024, "");
+};
+
+template <class T, class C>
+__global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void bwd_win_kernel(const BwdArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    uint16_t *sQ = reinterpret_cast<uint16_t *>(smem), *sdO = sQ + C::SQ, *sK = sdO + C::SDO, *sdS = sK + C::SK;
+    float *sStat = reinterpret_cast<float *>(sdS + C::SDS);
+    // (LDS byte addresses of the tiles for the copy instructions, taken here once from the array itself)
+    const uint32_t lds_q = lds_addr_of(smem), lds_do = lds_q + 2 * C::SQ, lds_k = lds_do + 2 * C::SDO;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    const int group = a.group > 1 ? a.group : 1;
+    const int nbg = (a.B + group - 1) / group;
+    const int work = xcd_remap(blockIdx.x, nbg * a.H);
+    const int bg = work / a.H, h = work % a.H;
+    const int wk0 = wave * 32; // first key of this wave
+    const int nb = wave & 3;   // phase 2: this wave's query block of the step
+
+    {   // clear LDS once: channel padding, and the dS rows of waves whose keys do not exist, are never written
+        u32x4_t *z = reinterpret_cast<u32x4_t *>(smem);
+        for (int i = tid; i < C::LDS_BYTES / 16; i += C::NTHREADS) z[i] = u32x4_t{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+
+    f32x16_t acc_dv[1][1], acc_dk[1][C::MB1], acc_dqb;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+#pragma unroll
+        for (int n = 0; n < C::MB1; ++n) acc_dk[0][n][v] = 0.f;
+        acc_dqb[v] = 0.f;
+    }
+
+    // the copies of a window: [Q | Q_b] and [K | K_b] (32 rows per wave each), dO (two instructions of 16 rows per wave)
+    TileDma<C::LQ, C::ROWCH, C::NWAVES, (C::NKR > 0)> cq;
+    TileDma<C::BN, C::ROWCH, C::NWAVES, (C::NKR > 0)> ck;
+    cq.init(a.q.ptr, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? a.qb.ptr : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane, 0);
+    ck.init(a.k.ptr, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? a.kb.ptr : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane, 0);
+    uint32_t do_off0, do_off1; // (rows past the end step back to the last one)
+    {
+        int row, chunk;
+        lean_copy_place<4>(lane, row, chunk);
+        do_off0 = (uint32_t)(min(32 * wave + row, a.Lq - 1) * (int)(a.dout.ss * 2) + chunk * 16);
+        do_off1 = (uint32_t)(min(32 * wave + 16 + row, a.Lq - 1) * (int)(a.dout.ss * 2) + chunk * 16);
+    }
+
+    const float to_log2 = C::FOLD ? a.scale * kLog2e : kLog2e;
+    const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
+    const bool visible = wk0 < a.Lk;
+
+    // What a window needs from global memory apart from its [K | K_b] tile, requested as early as the previous
+    // window allows: [Q | Q_b] and dO into their tiles (7 or 11 copy instructions per wave); K, K_b and V of this
+    // lane's key into registers (B operands of S and dP); and, for the per-query statistics, the two 16-channel
+    // halves of o and dO of query tid / 2 with its lse.
+    u32x4_t kreg[C::NK], vreg[C::NKD], so[2], sd[2];
+    float slse;
+#define FB_WIN_REQUEST(bexpr)                                                                                              \
+    {                                                                                                                      \
+        const int bq_ = __builtin_amdgcn_readfirstlane(bexpr);                                                             \
+        cq.pa = reinterpret_cast<const uint8_t *>(a.q.ptr + bq_ * a.q.sb + h * a.q.sh);                                    \
+        if constexpr (C::NKR > 0) cq.pb = reinterpret_cast<const uint8_t *>(a.qb.ptr + bq_ * a.qb.sb + h * a.qb.sh);       \
+        cq.issue(lds_q, 0, a.Lq, a.q.ss, C::NKR > 0 ? a.qb.ss : 0, 2 * C::NKD);                                            \
+        const uint16_t *dobase_ = a.dout.ptr + bq_ * a.dout.sb + h * a.dout.sh;                                            \
+        lds_dma16_all(do_off0, dobase_, lds_do + (2 * wave) * 1024);                                                       \
+        lds_dma16_all(do_off1, dobase_, lds_do + (2 * wave + 1) * 1024);                                                   \
+        const int key_ = wk0 + (threadIdx.x & 31), g_ = (threadIdx.x >> 5) & 1;                                            \
+        const uint16_t *kbase_ = a.k.ptr + bq_ * a.k.sb + h * a.k.sh, *vbase_ = a.v.ptr + bq_ * a.v.sb + h * a.v.sh;       \
+        _Pragma("unroll") for (int t = 0; t < C::NKD; ++t) {                                                               \
+            kreg[t] = load_chunk<true>(kbase_, a.k.ss, key_, a.Lk, 16 * t + 8 * g_, a.d);                                  \
+            vreg[t] = load_chunk<true>(vbase_, a.v.ss, key_, a.Lk, 16 * t + 8 * g_, a.d);                                  \
+        }                                                                                                                  \
+        if constexpr (C::NKR > 0) {                                                                                        \
+            const uint16_t *kbbase_ = a.kb.ptr + bq_ * a.kb.sb + h * a.kb.sh;                                              \
+            _Pragma("unroll") for (int t = 0; t < C::NKR; ++t)                                                             \
+                kreg[C::NKD + t] = load_chunk<true>(kbbase_, a.kb.ss, key_, a.Lk, 16 * t + 8 * g_, a.r);                   \
+        }                                                                                                                  \
+        const int rr_ = min((int)(threadIdx.x >> 1), a.Lq - 1), ch_ = 16 * (threadIdx.x & 1);                              \
+        const uint16_t *orow_ = a.o.ptr + bq_ * a.o.sb + h * a.o.sh + (int64_t)rr_ * a.o.ss + ch_;                         \
+        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                                    \
+            so[j] = *reinterpret_cast<const u32x4_t *>(orow_ + 8 * j);                                                     \
+            sd[j] = *reinterpret_cast<const u32x4_t *>(dobase_ + (int64_t)rr_ * a.dout.ss + ch_ + 8 * j);                  \
+        }                                                                                                                  \
+        slse = a.lse[((int64_t)bq_ * a.H + h) * a.Lq + rr_];                                                               \
+    }
+    if (bg * group < a.B) FB_WIN_REQUEST(bg * group)
+
+    for (int bi = 0; bi < group; ++bi) {
+        const int b = __builtin_amdgcn_readfirstlane(bg * group + bi);
+        if (b >= a.B) break;
+        int tid_again = threadIdx.x; // (opaque: what derives from the lane id is recomputed per window, not kept in registers)
+        asm volatile("" : "+v"(tid_again));
+        const int tid = tid_again, lane = tid & 63, c = lane & 31, g = lane >> 5;
+        const int key = wk0 + c;
+
+        // ---- this window.  Everything but its [K | K_b] tile was requested during the previous window (or above);
+        // every wave has left the previous window's [K | K_b] and dS tiles and its statistics (the barrier that
+        // ends a step).
+        {   // the per-query statistics (_bwd_preprocess_do_o_dot, flash_bias_triton.py:358-400): thread 2 i + j sums
+            // channels [16 j, 16 j + 16) of o * dO of query i, the pair adds up; lse * log2(e) and -delta go to LDS.
+            // Queries past the end get P = 0.
+            const int row = tid >> 1, half = tid & 1;
+            const bool ok = row < a.Lq;
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    sum = __builtin_fmaf(T::to_float((uint16_t)(so[j][e] & 0xffffu)), T::to_float((uint16_t)(sd[j][e] & 0xffffu)), sum);
+                    sum = __builtin_fmaf(T::to_float((uint16_t)(so[j][e] >> 16)), T::to_float((uint16_t)(sd[j][e] >> 16)), sum);
+                }
+            const float other = __shfl_xor(sum, 1, 64);
+            const float delta = half == 0 ? sum + other : other + sum; // (the same order in both lanes)
+            if (half == 0) {
+                sStat[row] = ok ? slse * kLog2e : INFINITY;
+                sStat[C::LQ + row] = ok ? -delta : 0.f;
+            }
+        }
+        ck.pa = reinterpret_cast<const uint8_t *>(a.k.ptr + b * a.k.sb + h * a.k.sh);
+        if constexpr (C::NKR > 0) ck.pb = reinterpret_cast<const uint8_t *>(a.kb.ptr + b * a.kb.sb + h * a.kb.sh);
+        // (loads return in order: with the statistics' inputs here, the tiles requested before them have landed;
+        // what this waits for beyond that are the few stores of the previous window's last step)
+        wait_vmcnt<0>();
+        ck.issue(lds_k, 0, a.Lk, a.k.ss, C::NKR > 0 ? a.kb.ss : 0, 2 * C::NKD); // (first read in phase 2)
+        barrier_lds();
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            acc_dv[0][0][v] = 0.f;
+            acc_dk[0][0][v] = 0.f; // (block 0 is dk; block 1, dk_bias, runs on over the group)
+        }
+        const uint32_t do_lds = lds_do;
+        const uint32_t do_row[2] = {do_lds + lean_row_addr<4>(c, g), do_lds + lean_row_addr<4>(c, 2 + g)};
+        const uint32_t do_col[2] = {do_lds + lean_tr_addr4(c, g, 0), do_lds + lean_tr_addr4(c, g, 1)};
+
+#pragma unroll 1
+        for (int step = 0; step < nsteps; ++step) {
+            const int m0 = step * C::BMQ;
+            // ---- phase 1: this wave's 32 keys against the step's 128 queries
+            if (visible) {
+#pragma unroll 1
+                for (int qb = 0; qb < C::QBLK; ++qb) {
+                    const int r0 = m0 + qb * 32;
+                    if (r0 >= a.Lq) break;
+                    u32x4_t qa[C::NK], da[C::NKD];
+#pragma unroll
+                    for (int t = 0; t < C::NK; ++t) qa[t] = *reinterpret_cast<const u32x4_t *>(sQ + swz_off<C::ROWCH>(r0 + c, 2 * t + g));
+#pragma unroll
+                    for (int t = 0; t < C::NKD; ++t) da[t] = lds_load16(do_row[t] + (r0 >> 5) * 2048);
+                    f32x16_t s, dp;
+                    float lse2[16];
+#pragma unroll
+                    for (int bq = 0; bq < 4; ++bq) { // register v <-> query r0 + 8 (v / 4) + 4 g + v % 4
+                        const f32x4_t l4 = *reinterpret_cast<const f32x4_t *>(sStat + r0 + 8 * bq + 4 * g);
+                        const f32x4_t d4 = *reinterpret_cast<const f32x4_t *>(sStat + C::LQ + r0 + 8 * bq + 4 * g);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            lse2[4 * bq + e] = l4[e];
+                            dp[4 * bq + e] = d4[e];
+                        }
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+                    for (int t = 0; t < C::NKD; ++t) s = T::mfma(qa[t], kreg[t], s);
+#pragma unroll
+                    for (int t = 0; t < C::NKD; ++t) dp = T::mfma(da[t], vreg[t], dp);
+                    if constexpr (!C::FOLD) { // the softmax scale multiplies q k^T only (flash_bias_triton.py:248)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) s[v] *= a.scale;
+                    }
+#pragma unroll
+                    for (int t = C::NKD; t < C::NK; ++t) s = T::mfma(qa[t], kreg[t], s);
+                    if (wk0 + 32 > a.Lk) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (key >= a.Lk) s[v] = -INFINITY;
+                    }
+                    u32x4_t pp[2], pds[2]; // P and dS, packed, per 16-query step
+#pragma unroll
+                    for (int v = 0; v < 16; v += 2) {
+                        const float p0 = fast_exp2(__builtin_fmaf(s[v], to_log2, -lse2[v]));
+                        const float p1 = fast_exp2(__builtin_fmaf(s[v + 1], to_log2, -lse2[v + 1]));
+                        pp[v >> 3][(v & 7) >> 1] = T::pack2(p0, p1);
+                        pds[v >> 3][(v & 7) >> 1] = T::pack2(p0 * dp[v], p1 * dp[v + 1]);
+                    }
+                    // dS of (this key, queries r0 + 16 t + 8 half + 4 g + 0..3) -> row `key` of the dS tile
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int half = 0; half < 2; ++half)
+                            *reinterpret_cast<u32x2_t *>(sdS + swz_off<C::ROWCHS>(key, 4 * qb + 2 * t + half) + 4 * g) =
+                                u32x2_t{pds[t][2 * half], pds[t][2 * half + 1]};
+                    // dV^T += dO^T P ; [dK | dK_b]^T += [Q | Q_b]^T dS  (contraction over this block's queries)
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        const u32x4_t dot = lds_load_tr(do_col[0] + ((r0 >> 4) + t) * 1024, do_col[1] + ((r0 >> 4) + t) * 1024);
+                        acc_dv[0][0] = T::mfma(dot, pp[t], acc_dv[0][0]);
+#pragma unroll
+                        for (int n = 0; n < C::MB1; ++n) {
+                            const u32x4_t qt = lds_read_a_tr<C::ROWCH>(sQ, r0 + 16 * t, 32 * n, c, g);
+                            acc_dk[0][n] = T::mfma(qt, pds[t], acc_dk[0][n]);
+                        }
+                    }
+                }
+            }
+            if (step == 0) wait_vmcnt<0>(); // this wave's share of the [K | K_b] tile has landed
+            barrier_lds(); // the step's dS tile is complete
+            if (step == nsteps - 1) {
+                // dv and dk (times scale) of this window are final, and nobody reads its [Q | Q_b] and dO tiles or needs
+                // K, K_b, V in registers any more: the next window's are requested now and arrive during phase 2
+                dkv_store<T, C, false>(a, acc_dv, acc_dk, b, h, wk0, c, g);
+                if (bi + 1 < group && b + 1 < a.B) FB_WIN_REQUEST(b + 1)
+            }
+            // ---- phase 2: one 32 x 32 block of [dQ | dQ_b]^T per wave, over all keys: queries m0 + 32 nb ..; the
+            // step's dq_bias blocks (channels 32 ..) go to waves 4 step .. 4 step + 3, its dq blocks to the other four
+            const bool bias_block = (wave >> 2) == step;
+            if ((!bias_block || C::BG) && m0 + 32 * nb < a.Lq) {
+                f32x16_t acc2;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc2[v] = bias_block ? acc_dqb[v] : 0.f;
+                const int col0 = bias_block ? 32 : 0;
+#pragma unroll 4
+                for (int key0 = 0; key0 < a.Lk; key0 += 16) {
+                    const u32x4_t ka = lds_read_a_tr<C::ROWCH>(sK, key0, col0, c, g);
+                    const u32x4_t db = lds_read_a_tr<C::ROWCHS>(sdS, key0, 32 * nb, c, g);
+                    acc2 = T::mfma(ka, db, acc2);
+                }
+                if (bias_block) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc_dqb[v] = acc2[v];
+                } else {
+                    const int query = m0 + 32 * nb + c;
+                    const bool ok = query < a.Lq;
+                    uint16_t *row = const_cast<uint16_t *>(a.dq.ptr) + b * a.dq.sb + h * a.dq.sh + (int64_t)(ok ? query : 0) * a.dq.ss;
+                    store_acc_rows<T, true>(row, ok, a.dq.vec_ok, acc2, a.scale, a.d, g);
+                }
+            }
+            barrier_lds(); // everyone has read the dS tile
+        }
+    }
+
+    // ---- the factor gradients, summed over the group's batch entries
+    if constexpr (C::BG) {
+        if (a.dkb.ptr) {
+            const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            const int c = lane_end & 31, g = lane_end >> 5;
+            dkv_store<T, C, true>(a, acc_dv, acc_dk, bg, h, wk0, c, g);
+            // this wave's dq_bias block: queries 128 (wave / 4) + 32 (wave % 4) ..
+            const int query = C::BMQ * (wave >> 2) + 32 * nb + c;
+            const bool ok = query < a.Lq;
+            uint16_t *row = const_cast<uint16_t *>(a.dqb.ptr) + bg * a.dqb.sb + h * a.dqb.sh + (int64_t)(ok ? query : 0) * a.dqb.ss;
+            store_acc_rows<T, true>(row, ok, a.dqb.vec_ok, acc_dqb, 1.f, a.r, g);
+        }
+    }
+}
+
+#undef FB_WIN_REQUEST
+
+template <class T, int NKR, bool FOLD, bool BG>
+static hipError_t launch_win_cfg(const BwdArgs &a, hipStream_t stream) {
+    typedef WinCfg<T, NKR, FOLD, BG> C;
+    auto kern = bwd_win_kernel<T, C>;
+    static KernelOnce once;
+    const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
+    if (e != hipSuccess) return e;
+    const int group = a.group > 1 ? a.group : 1;
+    return launch_flat(kern, (int64_t)((a.B + group - 1) / group) * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
+}
+
+template <class T, int NKR>
+static hipError_t launch_win_r(const BwdArgs &a, hipStream_t stream) {
+    const bool fold = a.r == 0 || a.scale == 1.f;
+    const bool bg = NKR > 0 && a.dqb.ptr;
+    if (fold) return bg ? launch_win_cfg<T, NKR, true, true>(a, stream) : launch_win_cfg<T, NKR, true, false>(a, stream);
+    return bg ? launch_win_cfg<T, NKR, false, true>(a, stream) : launch_win_cfg<T, NKR, false, false>(a, stream);
+}
+
+// Compiled once per element type for head dim 32 (see Makefile).  When fb_bwd takes this path is decided by
+// window_backward() in fb_kernels.h; the statistics must be in the scratch buffer (preprocess step).
+#define FB_CAT2(a, b) a##b
+#define FB_CAT(a, b) FB_CAT2(a, b)
+hipError_t FB_CAT(launch_bwd_win_, FB_SUFFIX)(const BwdArgs &a, hipStream_t stream) {
+    switch (nkr_of(a.r)) {
+    case 0: return launch_win_r<FB_T, 0>(a, stream);
+    case 1: return launch_win_r<FB_T, 1>(a, stream);
+    default: return launch_win_r<FB_T, 2>(a, stream);
+    }
+}
+
+} // namespace fb

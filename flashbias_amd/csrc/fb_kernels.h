@@ -114,6 +114,20 @@ inline bool mixed_backward(const BwdArgs &a0) {
     return ndq % 8 == 0 && ndkv % 8 == 0 && ndq <= num_cus() && ndkv <= num_cus();
 }
 
+// Whether fb_bwd runs the window kernel (fb_bwd_win.hip: one workgroup per (batch, head) forms the per-query
+// statistics and all five gradients, dq summed inside the workgroup) instead of the dq and dk/dv launches: whole
+// sequences of at most 256 positions, head dim 32, rank a multiple of 8 up to 32, aligned tensors, no additive or
+// causal mask, and at least one workgroup per compute unit (a workgroup fills a compute unit by itself).  Such
+// sequences are bound by memory traffic, and the two-kernel backward reads q, k, v, o and dO twice.
+inline bool window_backward(const BwdArgs &a) {
+    const int64_t lim = (int64_t)1 << 22; // (32-bit byte offsets of 256 tile rows)
+    const int group = a.group > 1 ? a.group : 1;
+    return a.mask.type == 0 && !a.causal && a.d == 32 && a.r % 8 == 0 && a.r <= 32 && a.Lq <= 256 && a.Lk <= 256 &&
+           a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.o.vec_ok && a.dout.vec_ok && (a.r == 0 || (a.qb.vec_ok && a.kb.vec_ok)) &&
+           a.q.ss < lim && a.k.ss < lim && a.dout.ss < lim && (a.r == 0 || (a.qb.ss < lim && a.kb.ss < lim)) &&
+           (int64_t)((a.B + group - 1) / group) * a.H >= num_cus();
+}
+
 // What a launcher remembers about one kernel instantiation (one static object per instantiation;
 // the only mutable state of the library besides num_cus() and fb_bwd_static's scratch address:
 // write-once values, atomics, so concurrent first calls from several threads are fine).
