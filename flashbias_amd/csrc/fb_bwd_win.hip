@@ -80,58 +80,97 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         acc_dqb[v] = 0.f;
     }
 
-    // the copies of a window: [Q | Q_b] and [K | K_b] (32 rows per wave each), dO (two instructions of 16 rows per wave)
-    TileDma<C::LQ, C::ROWCH, C::NWAVES, (C::NKR > 0)> cq;
-    TileDma<C::BN, C::ROWCH, C::NWAVES, (C::NKR > 0)> ck;
+    // The copies of a window, in halves of 128 rows so that a half can be refilled as soon as its step is over: per
+    // half and wave two instructions (16 rows) of Q, two of Q_b, two of K, two of K_b and one (16 rows) of dO.
+    typedef TileDma<128, C::ROWCH, C::NWAVES, (C::NKR > 0)> Copy;
+    Copy cq;
     cq.init(a.q.ptr, a.q.ss, a.d, 2 * C::NKD, C::NKR > 0 ? a.qb.ptr : nullptr, C::NKR > 0 ? a.qb.ss : 0, a.r, wave, lane, 0);
-    ck.init(a.k.ptr, a.k.ss, a.d, 2 * C::NKD, C::NKR > 0 ? a.kb.ptr : nullptr, C::NKR > 0 ? a.kb.ss : 0, a.r, wave, lane, 0);
-    uint32_t do_off0, do_off1; // (rows past the end step back to the last one)
+    uint32_t do_off[2]; // (rows past the end step back to the last one)
     {
         int row, chunk;
         lean_copy_place<4>(lane, row, chunk);
-        do_off0 = (uint32_t)(min(32 * wave + row, a.Lq - 1) * (int)(a.dout.ss * 2) + chunk * 16);
-        do_off1 = (uint32_t)(min(32 * wave + 16 + row, a.Lq - 1) * (int)(a.dout.ss * 2) + chunk * 16);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+            do_off[hf] = (uint32_t)(min(128 * hf + 16 * wave + row, a.Lq - 1) * (int)(a.dout.ss * 2) + chunk * 16);
     }
+    // One tensor's two instructions for rows [128 hf, 128 hf + 128) of a [X | X_b] tile (second: the factor part).
+    auto copy_half = [&](const Copy &cp, const uint16_t *base, int64_t ld, uint32_t lds_tile, int hf, int nrows, bool second) {
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(base) + (int64_t)(128 * hf) * ld * 2;
+#pragma unroll
+        for (int j = 0; j < Copy::NI; ++j) {
+            uint32_t off = cp.off[j];
+            if (128 * hf + 128 > nrows) { // a ragged half: rows past the end re-read the last row
+                const int r = ((wave * Copy::NI + j) * 64 + (int)(threadIdx.x & 63)) / C::ROWCH;
+                off -= (uint32_t)max(128 * hf + r - (nrows - 1), 0) * (uint32_t)(ld * 2);
+            }
+            // (the LDS address is wave-uniform; said again for the compiler, which must hand the copy a scalar)
+            const uint32_t dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_tile + hf * 16384 + (wave * Copy::NI + j) * 1024));
+            lds_dma16_lanes(off, src, dst, second ? cp.lanes_b[j] : cp.lanes_a[j]);
+        }
+    };
 
     const float to_log2 = C::FOLD ? a.scale * kLog2e : kLog2e;
     const int nsteps = (a.Lq + C::BMQ - 1) / C::BMQ;
     const bool visible = wk0 < a.Lk;
 
-    // What a window needs from global memory apart from its [K | K_b] tile, requested as early as the previous
-    // window allows: [Q | Q_b] and dO into their tiles (7 or 11 copy instructions per wave); K, K_b and V of this
-    // lane's key into registers (B operands of S and dP); and, for the per-query statistics, the two 16-channel
-    // halves of o and dO of query tid / 2 with its lse.
-    u32x4_t kreg[C::NK], vreg[C::NKD], so[2], sd[2];
+    // What a window needs from global memory, requested piece by piece while the previous window computes (a wave
+    // that issues many copies at once waits for the memory pipeline to take them):
+    //   queries(b, hf, part): rows [128 hf, 128 hf + 128) of Q (part 0), Q_b (1), dO (2) into their tiles
+    //   operands(b):          K, K_b and V of this lane's key into registers (B operands of S and dP; the [K | K_b] tile
+    //                         that phase 2 reads column-wise is written from them)
+    //   stat_inputs(b):       for the statistics of the 32 queries whose dO rows this wave copies: 16 channels of o
+    //                         per lane, and the lse
+    u32x4_t kreg[C::NK], vreg[C::NKD], so[2];
     float slse;
-#define FB_WIN_REQUEST(bexpr)                                                                                              \
-    {                                                                                                                      \
-        const int bq_ = __builtin_amdgcn_readfirstlane(bexpr);                                                             \
-        cq.pa = reinterpret_cast<const uint8_t *>(a.q.ptr + bq_ * a.q.sb + h * a.q.sh);                                    \
-        if constexpr (C::NKR > 0) cq.pb = reinterpret_cast<const uint8_t *>(a.qb.ptr + bq_ * a.qb.sb + h * a.qb.sh);       \
-        cq.issue(lds_q, 0, a.Lq, a.q.ss, C::NKR > 0 ? a.qb.ss : 0, 2 * C::NKD);                                            \
-        const uint16_t *dobase_ = a.dout.ptr + bq_ * a.dout.sb + h * a.dout.sh;                                            \
-        lds_dma16_all(do_off0, dobase_, lds_do + (2 * wave) * 1024);                                                       \
-        lds_dma16_all(do_off1, dobase_, lds_do + (2 * wave + 1) * 1024);                                                   \
-        const int key_ = wk0 + (threadIdx.x & 31), g_ = (threadIdx.x >> 5) & 1;                                            \
-        const uint16_t *kbase_ = a.k.ptr + bq_ * a.k.sb + h * a.k.sh, *vbase_ = a.v.ptr + bq_ * a.v.sb + h * a.v.sh;       \
-        _Pragma("unroll") for (int t = 0; t < C::NKD; ++t) {                                                               \
-            kreg[t] = load_chunk<true>(kbase_, a.k.ss, key_, a.Lk, 16 * t + 8 * g_, a.d);                                  \
-            vreg[t] = load_chunk<true>(vbase_, a.v.ss, key_, a.Lk, 16 * t + 8 * g_, a.d);                                  \
-        }                                                                                                                  \
-        if constexpr (C::NKR > 0) {                                                                                        \
-            const uint16_t *kbbase_ = a.kb.ptr + bq_ * a.kb.sb + h * a.kb.sh;                                              \
-            _Pragma("unroll") for (int t = 0; t < C::NKR; ++t)                                                             \
-                kreg[C::NKD + t] = load_chunk<true>(kbbase_, a.kb.ss, key_, a.Lk, 16 * t + 8 * g_, a.r);                   \
-        }                                                                                                                  \
-        const int rr_ = min((int)(threadIdx.x >> 1), a.Lq - 1), ch_ = 16 * (threadIdx.x & 1);                              \
-        const uint16_t *orow_ = a.o.ptr + bq_ * a.o.sb + h * a.o.sh + (int64_t)rr_ * a.o.ss + ch_;                         \
-        _Pragma("unroll") for (int j = 0; j < 2; ++j) {                                                                    \
-            so[j] = *reinterpret_cast<const u32x4_t *>(orow_ + 8 * j);                                                     \
-            sd[j] = *reinterpret_cast<const u32x4_t *>(dobase_ + (int64_t)rr_ * a.dout.ss + ch_ + 8 * j);                  \
-        }                                                                                                                  \
-        slse = a.lse[((int64_t)bq_ * a.H + h) * a.Lq + rr_];                                                               \
+    // the query whose statistics this lane helps with: one of the rows of dO that its wave copies (16 of each half)
+    const int srow = 128 * (lane >> 5) + 16 * wave + ((lane >> 1) & 15);
+    auto queries = [&](int b, int hf, int part) {
+        if (128 * hf >= a.Lq) return;
+        if (part == 0) copy_half(cq, a.q.ptr + b * a.q.sb + h * a.q.sh, a.q.ss, lds_q, hf, a.Lq, false);
+        if constexpr (C::NKR > 0) {
+            if (part == 1) copy_half(cq, a.qb.ptr + b * a.qb.sb + h * a.qb.sh, a.qb.ss, lds_q, hf, a.Lq, true);
+        }
+        if (part == 2) {
+            // (wave-uniform by construction; said again for the compiler, which must hand the copy a scalar base)
+            const uint64_t db = reinterpret_cast<uint64_t>(a.dout.ptr + b * a.dout.sb + h * a.dout.sh);
+            const void *dobase = reinterpret_cast<const void *>(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(db >> 32)) << 32) |
+                                                                (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)db));
+            lds_dma16_all(do_off[hf], dobase, (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_do + (8 * hf + wave) * 1024)));
+        }
+    };
+    // (plain loads, nothing that would make the wave wait for them here: keys past the end read the last key, whose
+    // scores are hidden later, and factor channels past the rank read chunk 0 and are cleared where the window starts)
+    auto operands = [&](int b) {
+        const int key = min(wk0 + (int)(threadIdx.x & 31), a.Lk - 1), g = (threadIdx.x >> 5) & 1;
+        const uint16_t *krow = a.k.ptr + b * a.k.sb + h * a.k.sh + (int64_t)key * a.k.ss + 8 * g;
+        const uint16_t *vrow = a.v.ptr + b * a.v.sb + h * a.v.sh + (int64_t)key * a.v.ss + 8 * g;
+#pragma unroll
+        for (int t = 0; t < C::NKD; ++t) {
+            kreg[t] = *reinterpret_cast<const u32x4_t *>(krow + 16 * t);
+            vreg[t] = *reinterpret_cast<const u32x4_t *>(vrow + 16 * t);
+        }
+        if constexpr (C::NKR > 0) {
+            const uint16_t *kbrow = a.kb.ptr + b * a.kb.sb + h * a.kb.sh + (int64_t)key * a.kb.ss;
+#pragma unroll
+            for (int t = 0; t < C::NKR; ++t) kreg[C::NKD + t] = *reinterpret_cast<const u32x4_t *>(kbrow + (16 * t + 8 * g < a.r ? 16 * t + 8 * g : 0));
+        }
+    };
+    auto stat_inputs = [&](int b) {
+        const int rr = min(srow, a.Lq - 1), ch = 16 * (threadIdx.x & 1);
+        const uint16_t *orow = a.o.ptr + b * a.o.sb + h * a.o.sh + (int64_t)rr * a.o.ss + ch;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) so[j] = *reinterpret_cast<const u32x4_t *>(orow + 8 * j);
+        slse = a.lse[((int64_t)b * a.H + h) * a.Lq + rr];
+    };
+    if (bg * group < a.B) { // the first window of the workgroup: everything at once
+        const int b0 = __builtin_amdgcn_readfirstlane(bg * group);
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+            for (int part = 0; part < 3; ++part) queries(b0, hf, part);
+        operands(b0);
+        stat_inputs(b0);
     }
-    if (bg * group < a.B) FB_WIN_REQUEST(bg * group)
 
     for (int bi = 0; bi < group; ++bi) {
         const int b = __builtin_amdgcn_readfirstlane(bg * group + bi);
@@ -141,35 +180,46 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         const int tid = tid_again, lane = tid & 63, c = lane & 31, g = lane >> 5;
         const int key = wk0 + c;
 
-        // ---- this window.  Everything but its [K | K_b] tile was requested during the previous window (or above);
-        // every wave has left the previous window's [K | K_b] and dS tiles and its statistics (the barrier that
-        // ends a step).
-        {   // the per-query statistics (_bwd_preprocess_do_o_dot, flash_bias_triton.py:358-400): thread 2 i + j sums
-            // channels [16 j, 16 j + 16) of o * dO of query i, the pair adds up; lse * log2(e) and -delta go to LDS.
+        // ---- this window.  The first half of its query-side tiles, its register operands and the inputs of its
+        // statistics were requested during the previous window (or above); every wave has left the previous window's
+        // [K | K_b] and dS tiles and its statistics (the barrier that ends a step).
+        const bool next = bi + 1 < group && b + 1 < a.B;
+        const int bn = __builtin_amdgcn_readfirstlane(b + 1);
+        // Everything requested for this window has landed (what this waits for beyond that are the few stores of the
+        // previous window's last step).
+        wait_vmcnt<0>();
+        {   // the per-query statistics (_bwd_preprocess_do_o_dot, flash_bias_triton.py:358-400) of the 32 queries whose dO
+            // rows this wave copied itself (so that it may read them without a barrier): lanes 2 i and 2 i + 1 sum the
+            // channels [0, 16) and [16, 32) of o * dO of one query and add up; lse * log2(e) and -delta go to LDS.
             // Queries past the end get P = 0.
-            const int row = tid >> 1, half = tid & 1;
-            const bool ok = row < a.Lq;
+            const int half = tid & 1;
+            const bool ok = srow < a.Lq;
             float sum = 0.f;
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
+            for (int j = 0; j < 2; ++j) {
+                const u32x4_t sd = lds_load16(lds_do + lean_chunk_off<4>(srow, 2 * half + j));
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    sum = __builtin_fmaf(T::to_float((uint16_t)(so[j][e] & 0xffffu)), T::to_float((uint16_t)(sd[j][e] & 0xffffu)), sum);
-                    sum = __builtin_fmaf(T::to_float((uint16_t)(so[j][e] >> 16)), T::to_float((uint16_t)(sd[j][e] >> 16)), sum);
+                    sum = __builtin_fmaf(T::to_float((uint16_t)(so[j][e] & 0xffffu)), T::to_float((uint16_t)(sd[e] & 0xffffu)), sum);
+                    sum = __builtin_fmaf(T::to_float((uint16_t)(so[j][e] >> 16)), T::to_float((uint16_t)(sd[e] >> 16)), sum);
                 }
+            }
             const float other = __shfl_xor(sum, 1, 64);
             const float delta = half == 0 ? sum + other : other + sum; // (the same order in both lanes)
             if (half == 0) {
-                sStat[row] = ok ? slse * kLog2e : INFINITY;
-                sStat[C::LQ + row] = ok ? -delta : 0.f;
+                sStat[srow] = ok ? slse * kLog2e : INFINITY;
+                sStat[C::LQ + srow] = ok ? -delta : 0.f;
             }
         }
-        ck.pa = reinterpret_cast<const uint8_t *>(a.k.ptr + b * a.k.sb + h * a.k.sh);
-        if constexpr (C::NKR > 0) ck.pb = reinterpret_cast<const uint8_t *>(a.kb.ptr + b * a.kb.sb + h * a.kb.sh);
-        // (loads return in order: with the statistics' inputs here, the tiles requested before them have landed;
-        // what this waits for beyond that are the few stores of the previous window's last step)
-        wait_vmcnt<0>();
-        ck.issue(lds_k, 0, a.Lk, a.k.ss, C::NKR > 0 ? a.kb.ss : 0, 2 * C::NKD); // (first read in phase 2)
+        // the [K | K_b] tile, row `key` from this lane's register operands (factor channels past the rank cleared
+        // first; keys past the end hold the last key, whose dS is zero)
+        if constexpr (C::NKR > 0) {
+#pragma unroll
+            for (int t = 0; t < C::NKR; ++t)
+                if (16 * t + 8 * g >= a.r) kreg[C::NKD + t] = u32x4_t{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int t = 0; t < C::NK; ++t) *reinterpret_cast<u32x4_t *>(sK + swz_off<C::ROWCH>(key, 2 * t + g)) = kreg[t];
         barrier_lds();
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
@@ -184,11 +234,14 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         for (int step = 0; step < nsteps; ++step) {
             const int m0 = step * C::BMQ;
             // ---- phase 1: this wave's 32 keys against the step's 128 queries
-            if (visible) {
+            {
 #pragma unroll 1
                 for (int qb = 0; qb < C::QBLK; ++qb) {
                     const int r0 = m0 + qb * 32;
-                    if (r0 >= a.Lq) break;
+                    // a slice of the copies that may run now: during the second step the first half of the next window's
+                    // query-side tiles (its rows are no longer read)
+                    if (step == 1 && next && qb < 3) queries(bn, 0, qb);
+                    if (!visible || r0 >= a.Lq) continue;
                     u32x4_t qa[C::NK], da[C::NKD];
 #pragma unroll
                     for (int t = 0; t < C::NK; ++t) qa[t] = *reinterpret_cast<const u32x4_t *>(sQ + swz_off<C::ROWCH>(r0 + c, 2 * t + g));
@@ -223,6 +276,10 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                         for (int v = 0; v < 16; ++v)
                             if (key >= a.Lk) s[v] = -INFINITY;
                     }
+                    // (The vector instructions below read what the matrix instructions above have just written, which
+                    // takes wait states that the compiler inserts along straight-line code; here the two can meet
+                    // across the loop's branches, where it was seen to leave them out: they are spelt out.)
+                    asm volatile("s_nop 11" : "+v"(s), "+v"(dp));
                     u32x4_t pp[2], pds[2]; // P and dS, packed, per 16-query step
 #pragma unroll
                     for (int v = 0; v < 16; v += 2) {
@@ -251,14 +308,20 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                     }
                 }
             }
-            if (step == 0) wait_vmcnt<0>(); // this wave's share of the [K | K_b] tile has landed
             barrier_lds(); // the step's dS tile is complete
             if (step == nsteps - 1) {
-                // dv and dk (times scale) of this window are final, and nobody reads its [Q | Q_b] and dO tiles or needs
-                // K, K_b, V in registers any more: the next window's are requested now and arrive during phase 2
+                // dv and dk (times scale) of this window are final and K, K_b, V in registers no longer needed: the
+                // next window's are requested now and arrive during phase 2
                 dkv_store<T, C, false>(a, acc_dv, acc_dk, b, h, wk0, c, g);
-                if (bi + 1 < group && b + 1 < a.B) FB_WIN_REQUEST(b + 1)
+                if (next) {
+                    operands(bn);
+                    // the rows of the second half of the query-side tiles are free as well (with a single step: those
+                    // of the first half, which had no second step to be spread over)
+#pragma unroll
+                    for (int part = 0; part < 3; ++part) queries(bn, nsteps == 1 ? 0 : 1, part);
+                }
             }
+            if (step == 0 && next) stat_inputs(bn);
             // ---- phase 2: one 32 x 32 block of [dQ | dQ_b]^T per wave, over all keys: queries m0 + 32 nb ..; the
             // step's dq_bias blocks (channels 32 ..) go to waves 4 step .. 4 step + 3, its dq blocks to the other four
             const bool bias_block = (wave >> 2) == step;
@@ -273,6 +336,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
                     const u32x4_t db = lds_read_a_tr<C::ROWCHS>(sdS, key0, 32 * nb, c, g);
                     acc2 = T::mfma(ka, db, acc2);
                 }
+                asm volatile("s_nop 11" : "+v"(acc2)); // (as above: the loop's exit lies between the last product and its first reader)
                 if (bias_block) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) acc_dqb[v] = acc2[v];
@@ -301,8 +365,6 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         }
     }
 }
-
-#undef FB_WIN_REQUEST
 
 template <class T, int NKR, bool FOLD, bool BG>
 static hipError_t launch_win_cfg(const BwdArgs &a, hipStream_t stream) {
