@@ -18,6 +18,7 @@ evaluated on the very tensors of the timed steps: a subset of query rows against
 plus the size-independent checksums), ``sweep`` (forward and forward + backward milliseconds of
 every benchmark configuration at its stated size, timed through ``flash_bias_func`` and autograd,
 so that gradient reduction over broadcast factors, rank padding and mask folding are inside),
+``modules`` (forward and forward + backward milliseconds of the two module drop-ins, projections included),
 ``fp16`` (the headline step in fp16, the dtype of the reference's published numbers),
 ``factors_permuted_inside`` (the headline step with the (B, H, L, r) -> (B, L, H, r)
 ``permute().contiguous()`` of the factors inside the timed region, as flash_bias/benchmark.py:233-235
@@ -40,16 +41,16 @@ PEAK_HBM_GBS = 8000.0
 PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "headline_fwd_bwd_kernels.md")
 
 
-def _profiled_traffic(kernel):
-    """HBM bytes per launch of `kernel` at the headline shape as the tracked rocprofv3 summary states
-    them (a line `hbm_bytes_per_launch <kernel> <bytes>`: FETCH_SIZE and WRITE_SIZE counters scaled
-    by a copy of known size); None when the summary has no such line.  A counter figure, not
-    measured live."""
+def _profiled(key, kernel):
+    """A figure of `kernel` at the headline shape as the tracked rocprofv3 summary states it, a line
+    `<key> <kernel> <value>`: `hbm_bytes_per_launch` (FETCH_SIZE and WRITE_SIZE counters scaled by a copy
+    of known size) or `avg_launch_ns` (the kernel trace's average duration); None when the summary has no
+    such line.  Figures of the profiled run, not measured live."""
     try:
         with open(PROFILE_SUMMARY) as f:
             for line in f:
                 parts = line.split()
-                if len(parts) >= 3 and parts[0] == "hbm_bytes_per_launch" and parts[1] == kernel:
+                if len(parts) >= 3 and parts[0] == key and parts[1] == kernel:
                     return float(parts[2])
     except OSError:
         pass
@@ -255,7 +256,8 @@ def _device_configs(dev):
         qb, kb = [(torch.randn(1, 768, 4, 32, device=dev) / math.sqrt(32)).bfloat16() for _ in range(2)]
         return q, k, v, qb, kb, do, False, 32
 
-    cfgs = [(f"sweep B2 H4 d32 r8 L={L}", lambda L=L: sweep(L)) for L in (1024, 2048, 4096, 8192, 16384)]
+    # (the reference's own sweep starts at 2^8, flash_bias/config.py:17)
+    cfgs = [(f"sweep B2 H4 d32 r8 L={L}", lambda L=L: sweep(L)) for L in (256, 512, 1024, 2048, 4096, 8192, 16384)]
     cfgs += [(f"alibi causal B1 H50 d32 r2 L={L}", lambda L=L: alibi(L)) for L in (2048, 4096, 8192)]
     cfgs += [("swin 4096 windows x 256 H16 d32 r16 (factors shared by the windows)", swin),
              ("pde N=32768 H8 d32 r5 (factors shared by the heads)", pde),
@@ -294,6 +296,35 @@ def _sweep(dev, steps, warmup, only=None):
                     "hbm_algorithmic_gb": round(hbm / 1e9, 3), "hbm_gbs": round(hbm / t_fb / 1e6, 1),
                     "pct_of_hbm_peak": round(100 * hbm / t_fb / 1e6 / PEAK_HBM_GBS, 2)})
         del q, k, v, qb, kb, do, leaves
+        torch.cuda.empty_cache()
+    return out
+
+
+def _modules(dev, steps, warmup):
+    """Layer-level timing of the two module drop-ins (flashbias_amd/modules.py) at the sizes of the benchmark
+    configurations they belong to: the ALiBi causal self-attention block
+    (1_Language_Model/attention_with_alibi_bias.py:18-64) at B1 L=4096 H50 x 32 and the Swin-V2 window attention
+    core (2_Vision_Transformer/swin_transformer_v2.py:155-207) on 4096 windows of 256 tokens, H16 x 32, rank 16.
+    bf16 parameters and activations, forward and forward + backward (gradient of the input and of every
+    parameter), the projections of the layer included."""
+    import torch
+    from flashbias_amd import modules
+    out = {}
+    cases = [("AttentionWithALiBiBias B1 L=4096 dim=1600 (H50 x 32), causal, exact rank-4 factors",
+              lambda: modules.AttentionWithALiBiBias(1600, 50, 32), (1, 4096, 1600)),
+             ("WindowAttentionCore 4096 windows x 256 tokens dim=512 (H16 x 32), rank 16",
+              lambda: modules.WindowAttentionCore(512, 16, 16, rank=16), (4096, 256, 512))]
+    for name, make, shape in cases:
+        torch.manual_seed(0)
+        mod = make().to(dev).to(torch.bfloat16)
+        x = torch.randn(*shape, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        dy = torch.randn(*shape, device=dev, dtype=torch.bfloat16)
+        params = [x] + [p for p in mod.parameters() if p.requires_grad]
+        with torch.no_grad():
+            t_fwd = _time_events(lambda: mod(x), steps, warmup)
+        t_fb = _time_events(lambda: torch.autograd.grad(mod(x), params, dy), steps, warmup)
+        out[name] = {"fwd_ms": round(t_fwd, 4), "fwd_bwd_ms": round(t_fb, 4)}
+        del mod, x, dy, params
         torch.cuda.empty_cache()
     return out
 
@@ -356,6 +387,9 @@ def headline(args):
     # the dQ|dQ_b product (d + r) and, beyond the algorithmic count, a second S / dP recompute.
     f_dkv = 2.0 * hl["B"] * hl["H"] * hl["L"] * hl["L"] * (4 * hl["d"] + 2 * hl["r"])
     tflops_main = f_dkv / (ms["fb_bwd_dkv"] * 1e-3) / 1e12
+    prof_ns = _profiled("avg_launch_ns", "bwd_dkv_lean_kernel")
+    prof_ms = None if prof_ns is None else round(prof_ns * 1e-6, 4)
+    prof_frac = None if prof_ns is None else round(f_dkv / (prof_ns * 1e-9) / 1e12 / PEAK_BF16_TFLOPS, 4)
     value = (f_fwd + f_bwd) / (ms_step * 1e-3) / 1e12
     ref_fwd, ref_fb = workloads.reference_formula_flops(hl["B"], hl["H"], hl["L"], hl["d"])
     out = {
@@ -379,9 +413,13 @@ def headline(args):
         "bwd_ms": round(ms["fb_bwd"], 4),
         "kernel_ms": {k: round(v, 4) for k, v in ms.items()},
         "reference_formula_tflops": round(ref_fb / (ms_step * 1e-3) / 1e12, 2),
+        # achieved / frac: this run's own launches (one event pair per launch on the launch stream).  The tracked
+        # profile's average for the same kernel (another box, under the profiler) is stated beside them.
         "roofline": {"kernel": "bwd_dkv_lean_kernel (fb_bwd_dkv)", "bound": "mfma", "achieved": round(tflops_main, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(tflops_main / PEAK_BF16_TFLOPS, 4),
-                     "traffic": _profiled_traffic("bwd_dkv_lean_kernel")},
+                     "traffic": _profiled("hbm_bytes_per_launch", "bwd_dkv_lean_kernel"),
+                     "flop_per_launch": f_dkv, "launch_ms": round(ms["fb_bwd_dkv"], 4),
+                     "profile_launch_ms": prof_ms, "frac_from_profile": prof_frac},
         "gate": gate,
     }
     del keep
@@ -412,6 +450,7 @@ def headline(args):
                             {"fwd_ms": round(den[0], 3), "fwd_bwd_ms": round(den[1], 3)}}
         torch.cuda.empty_cache()
         out["sweep"] = _sweep(dev, steps, warm)
+        out["modules"] = _modules(dev, steps, warm)
     if not args.no_cpu:
         out["cpu_baseline"] = _cpu_baseline(w, (f_fwd + f_bwd) / (hl["B"] * hl["H"]))
     print(json.dumps(out))
@@ -530,7 +569,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if args.only:
+    if args.only == "modules":
+        import torch
+        print(json.dumps({"modules": _modules(torch.device("cuda:0"), args.steps, args.warmup)}))
+    elif args.only:
         import torch
         print(json.dumps({"sweep": _sweep(torch.device("cuda:0"), args.steps, args.warmup, args.only)}))
     elif args.report:
