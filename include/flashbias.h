@@ -142,10 +142,15 @@ int fb_fwd(const fb_params *p, void *stream);
  * queries and leaves -delta and lse * log2(e) in the scratch buffer, then the key-stationary kernel
  * (dk, dv, dk_bias) that reads them.  (On grids that would give each of these kernels at most one
  * workgroup per compute unit: the preprocess phase, then a single launch that holds the workgroups of
- * both kernels side by side.)  The results are bit-identical to the three phases below
- * called one by one.  Unlike the reference there is no fp32 dq_accum buffer, no
- * atomics and no final cast (:1212-1219, :1340-1342): dq and dq_bias are accumulated in
- * registers by a query-stationary kernel and written once, so every gradient is
+ * both kernels side by side.)  The results of these are bit-identical to the three phases below
+ * called one by one.  Whole sequences of at most 256 positions (head dim 32, rank a multiple of 8 up to
+ * 32, aligned tensors, no additive or causal mask, at least one (batch, head) pair per compute unit: the
+ * window attention of swin_transformer_v2.py:178-203) take a single launch instead in which one
+ * workgroup forms delta and all five gradients of a (batch, head) pair, dq summed inside the workgroup;
+ * it leaves the scratch buffer untouched and its results equal the phases' up to the rounding of other
+ * summation orders.  Unlike the reference there is no fp32 dq_accum buffer, no atomics and no final
+ * cast on any of these paths (:1212-1219, :1340-1342): dq and dq_bias are accumulated in registers
+ * (or, for windows, in a fixed order through LDS) and written once, so every gradient is
  * bit-reproducible. */
 int fb_bwd(const fb_params *p, void *stream);
 
