@@ -122,8 +122,9 @@ int fb_check(const fb_params *p, int pass);
 /* The bias_grad_group this library recommends for a backward call: 1 unless both factors are shared by
  * the batch (stride_b = 0) and the call is a large batch of short sequences (the window attention of
  * swin_transformer_v2.py:178-203), where writing the full-shape factor gradients and summing them
- * afterwards costs more than the attention itself saves; then the largest of 8, 4, 2 that still
- * leaves every compute unit several workgroups.  Reads B, H, Lq, Lk, r and the factors' strides only.
+ * afterwards costs more than the attention itself saves; then the largest of 8, 4, 2 (32, 16, ... for whole
+ * sequences of at most 256 positions at head dim 32, which one workgroup per batch entry and head serves) that still
+ * leaves every compute unit several workgroups.  Reads the sizes, the causal flag, the mask type and the factors' strides only.
  * No counterpart in the reference. */
 int fb_suggest_bias_grad_group(const fb_params *p);
 

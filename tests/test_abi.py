@@ -137,7 +137,12 @@ def test_grouped_factor_gradients_checks_and_suggestion():
     p.B, p.H, p.Lq, p.Lk, p.r = 4096, 16, 256, 256, 16
     assert lib.fb_suggest_bias_grad_group(p) == 1      # the factors are not shared by the batch
     p.q_bias.stride_b = p.k_bias.stride_b = 0
+    assert lib.fb_suggest_bias_grad_group(p) == 32     # whole windows at head dim 32: one workgroup per (batch, head)
+    p.causal = 1
+    assert lib.fb_suggest_bias_grad_group(p) == 8      # ... which causal calls are not
+    p.causal, p.d = 0, 64
     assert lib.fb_suggest_bias_grad_group(p) == 8
+    p.d = 32
     p.B = 256
     assert lib.fb_suggest_bias_grad_group(p) == 4      # still 1024 workgroups of 256 queries
     p.B = 64
