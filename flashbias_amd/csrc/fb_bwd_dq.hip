@@ -470,7 +470,10 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
                     }
 #pragma unroll
                     for (int t = 0; t < C::NKD; ++t) dp = T::mfma(va[t], dor[qb][t], t == 0 ? negd[qb] : dp);
-                    const bool edge = (n0 + kb * 32 + 32 > a.Lk) || (a.causal && n0 + kb * 32 + 31 > wq0 + qb * 32);
+                    // (bitwise on purpose: a short-circuit evaluation puts a small block of scalar code between the last
+                    // MFMA and the branch, which the branch's other edge skips, and the compiler then counts the
+                    // wait states between an MFMA and the first reader of its result along the longer path only)
+                    const bool edge = (n0 + kb * 32 + 32 > a.Lk) | ((a.causal != 0) & (n0 + kb * 32 + 31 > wq0 + qb * 32));
                     if (edge) {
                         int key0 = n0 + kb * 32 + 4 * g;
                         asm volatile("" : "+v"(key0)); // (computed here, not kept in 16 registers across the loop)
