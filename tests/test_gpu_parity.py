@@ -641,6 +641,75 @@ def test_window_backward(gpu_device, dtype, B, H, Lq, Lk, r, scale, group, grads
             assert errors(got, want)[1] <= max(tol, GRAD_TOL), name
 
 
+def _random_windows(count, seed):
+    """Reproducible draws from what the window backward accepts: any lengths up to 256, ranks 0 ... 32 in steps of
+    8, both element types, factors per entry or shared with groups of any size, with or without factor gradients,
+    on grids of at least one workgroup per compute unit."""
+    import random
+    rnd = random.Random(seed)
+    out = []
+    for idx in range(count):
+        r = rnd.choice([0, 8, 16, 16, 24, 32])
+        group = rnd.choice([1, 1, 2, 3, 5, 8, 32]) if r else 1
+        H = rnd.choice([1, 2, 4, 8])
+        B = -(-rnd.choice([256, 300, 512]) // H) * group + rnd.choice([0, 0, 1, group - 1])
+        lens = [rnd.choice([1, 31, 32, 33, 64, 100, 127, 128, 129, 160, 200, 255, 256]) for _ in range(2)]
+        if rnd.random() < 0.4:
+            lens[1] = lens[0]
+        out.append((rnd.choice([torch.bfloat16, torch.float16]), B, H, lens[0], lens[1], r,
+                    rnd.choice([None, None, 1.0, 0.3]), group, rnd.random() < 0.7, idx))
+    return out
+
+
+@pytest.mark.parametrize("dtype,B,H,Lq,Lk,r,scale,group,grads,idx",
+                         _random_windows(int(os.environ.get("FB_RANDOM_WINDOWS", "10")),
+                                         int(os.environ.get("FB_RANDOM_SEED", "20240"))))
+def test_random_windows(gpu_device, dtype, B, H, Lq, Lk, r, scale, group, grads, idx):
+    """The window backward on shapes nobody picked by hand, against the three phases launched one by one (whose
+    kernels the rest of this file holds against the oracle) and against itself."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _params, _stream, _tensor
+    dev = gpu_device
+    g = torch.Generator(device="cpu").manual_seed(3000 + idx)
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(dtype).to(dev)
+    q, k, v, do = mk(B, Lq, H, 32), mk(B, Lk, H, 32), mk(B, Lk, H, 32), mk(B, Lq, H, 32)
+    qb = kb = None
+    if r:
+        fb = 1 if group > 1 else B
+        qb, kb = mk(fb, Lq, H, r) / r ** 0.5, mk(fb, Lk, H, r) / r ** 0.5
+    lib = _lib.load()
+
+    def run(fused):
+        p, keep = _params(q, k, v, qb, kb, None, False, scale)
+        bufs = dict(o=torch.empty_like(q), lse=torch.empty((B, H, Lq), device=dev, dtype=torch.float32),
+                    dq=torch.full_like(q, float("nan")), dk=torch.full_like(k, float("nan")), dv=torch.full_like(v, float("nan")),
+                    scratch=torch.empty(lib.fb_bwd_workspace_bytes(p) // 4, device=dev, dtype=torch.float32))
+        p.o, p.lse, p.dout = _tensor(bufs["o"]), bufs["lse"].data_ptr(), _tensor(do)
+        p.dq, p.dk, p.dv, p.delta = _tensor(bufs["dq"]), _tensor(bufs["dk"]), _tensor(bufs["dv"]), bufs["scratch"].data_ptr()
+        if r and grads:
+            rows = -(-B // group)
+            bufs["dqb"] = torch.full((rows, Lq, H, r), float("nan"), device=dev, dtype=dtype)
+            bufs["dkb"] = torch.full((rows, Lk, H, r), float("nan"), device=dev, dtype=dtype)
+            p.dq_bias, p.dk_bias = _tensor(bufs["dqb"]), _tensor(bufs["dkb"])
+        p.bias_grad_group = group if r else 0
+        _lib.check_status(lib.fb_fwd(p, _stream()))
+        for fn in ((lib.fb_bwd,) if fused else (lib.fb_bwd_preprocess, lib.fb_bwd_dkv, lib.fb_bwd_dq)):
+            _lib.check_status(fn(p, _stream()))
+        torch.cuda.synchronize()
+        del keep
+        return bufs
+
+    one, two, phases = run(True), run(True), run(False)
+    for name in ["dq", "dk", "dv"] + (["dqb", "dkb"] if r and grads else []):
+        a, b = one[name].float(), phases[name].float()
+        assert torch.isfinite(a).all(), name
+        assert torch.equal(one[name], two[name]), name
+        # (other kernels, other summation orders; grouped rows are sums of up to `group` entries rounded once; with a
+        # single key dq and dk are zero up to the rounding of the stored o, hence the floor)
+        scale_of = max(float(b.abs().max()), 0.05)
+        assert (a - b).abs().max() <= 2.0 ** -6 * scale_of, (name, float((a - b).abs().max()), float(b.abs().max()))
+
+
 def test_shared_factors_large_batch_of_windows(gpu_device):
     """A batch large enough for the library to suggest groups (64 windows x 16 heads of 256 tokens,
     factors shared by the windows, as in swin_transformer_v2.py:178-203): all five gradients through
