@@ -36,19 +36,6 @@ def _checksums(do, grads):
     assert gk.sum(1).abs().max() <= bound
 
 
-def _rows_on_cpu(rows, q, k, v, qb, kb, causal, scale, do):
-    """Oracle results (o, dq, dq_bias) for the given query rows against all keys; a causal mask
-    becomes an explicit additive mask of the rows' true positions."""
-    f = lambda t: t.detach().float().cpu()
-    sub = lambda t: f(t[:, rows])
-    mask = None
-    if causal:
-        hidden = torch.arange(k.shape[1])[None, :] > rows[:, None]
-        mask = torch.zeros(1, 1, len(rows), k.shape[1]).masked_fill(hidden[None, None], float("-inf"))
-    res = eager.flashbias_eager_grads(sub(q), f(k), f(v), sub(qb), f(kb), mask, False, scale, sub(do))
-    return res[0], res[1], res[4]
-
-
 def _heads_on_gpu(q, k, v, qb, kb, causal, scale, do, chunk):
     """The eager oracle in fp32 on the GPU, `chunk` heads at a time (batch of one); factors shared by
     the heads get their gradients summed over all chunks."""

@@ -45,6 +45,7 @@ def test_static_scratch_backward_matches_fb_bwd(gpu_device):
 
     run(2, 777, 3, 32, 8, True, seed=21)
     run(1, 130, 2, 32, 8, False, seed=22)  # smaller: the array still holds the first call's values
+    run(40, 200, 8, 32, 16, False, seed=24)  # whole sequences in one workgroup: a single launch that needs no scratch
 
 
 @pytest.mark.gpu
