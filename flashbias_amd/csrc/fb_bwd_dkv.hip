@@ -299,9 +299,8 @@ __device__ __forceinline__ void bwd_dkv_body(const BwdArgs &a, int wg) {
     const int group = a.group > 1 ? a.group : 1;
     const int nbg = (a.B + group - 1) / group;
     const int total = a.ntiles_n * nbg * a.H;
-    const int work = xcd_remap(wg, total);
-    const int bgh = work / a.ntiles_n;
-    const int tile_n = work % a.ntiles_n; // causal: low key tiles see the most queries, they go first
+    int bgh, tile_n; // (causal: the first key tile sees the most queries)
+    work_order(wg, a.ntiles_n, total, a.causal, bgh, tile_n);
     const int bg = bgh / a.H, h = bgh % a.H;
     const int n0 = tile_n * C::BN;
     const int wk0 = n0 + wave * (32 * C::KBW); // first key of this wave

@@ -65,9 +65,8 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_n * a.B * a.H;
-    const int work = xcd_remap(wg, total);
-    const int bh = work / a.ntiles_n;
-    const int tile_n = work % a.ntiles_n; // causal: low key tiles see the most queries, they go first
+    int bh, tile_n; // (causal: the first key tile sees the most queries)
+    work_order(wg, a.ntiles_n, total, a.causal, bh, tile_n);
     const int b = bh / a.H, h = bh % a.H;
     const int n0 = tile_n * C::BN;
     const int key = n0 + 32 * wave + c; // this lane's key

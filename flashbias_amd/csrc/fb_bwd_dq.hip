@@ -222,10 +222,9 @@ __device__ __forceinline__ void bwd_dq_body(const BwdArgs &a, int wg) {
     const int group = a.group > 1 ? a.group : 1;
     const int nbg = (a.B + group - 1) / group;
     const int total = a.ntiles_m * nbg * a.H;
-    const int work = xcd_remap(wg, total);
-    const int bgh = work / a.ntiles_m;
-    int tile_m = work % a.ntiles_m;
-    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
+    int bgh, tile_m;
+    work_order(wg, a.ntiles_m, total, a.causal, bgh, tile_m);
+    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // the last query tile sees the most keys
     const int bg = bgh / a.H, h = bgh % a.H;
     const int m0 = tile_m * C::BM;
     const int wq0 = m0 + wave * (32 * C::QBLK);
@@ -560,16 +559,16 @@ static hipError_t launch_dq_qb(const BwdArgs &a, hipStream_t stream) {
     return launch_dq_qb_bg<T, NKD, NKR, VEC, MASK, QB2, FOLD, KB1, true>(a, stream);
 }
 
-// 256-query workgroups (two blocks per wave) once every compute unit has two of them (four under
-// a causal mask: B1 H50 d32 at L=4096 is 11 % faster with the small ones, equal at L=8192, 3 %
-// slower at L=16384), 128-query workgroups below that and for short sequences whose last 256-query
+// 256-query workgroups (two blocks per wave) once every compute unit has two of them (three under
+// a causal mask: B1 H50 d32 r16 at L=4096 0.162 -> 0.153 ms with the large ones, equal at L=8192 and
+// L=16384), 128-query workgroups below that and for short sequences whose last 256-query
 // workgroup would be half empty (8192 x 16 windows of 128 tokens: 2.59 -> 1.76 ms): as in the forward
 // launcher.
 template <class T, int NKD, int NKR, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_dq_vec(const BwdArgs &a, hipStream_t stream) {
     if constexpr (DqCfg<T, NKD, NKR, VEC, MASK, true>::QBLK == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (wgs < (int64_t)(a.causal ? 4 : 2) * num_cus() || half_empty_256(a.Lq))
+        if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus() || half_empty_256(a.Lq))
             return launch_dq_qb<T, NKD, NKR, VEC, MASK, false, FOLD>(a, stream);
     }
     // head dims above 64, aligned, unmasked, rank <= 32: 32-key tiles fit two workgroups per CU

@@ -60,10 +60,9 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_m * a.B * a.H;
-    const int work = xcd_remap(wg, total);
-    const int bh = work / a.ntiles_m;
-    int tile_m = work % a.ntiles_m;
-    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
+    int bh, tile_m;
+    work_order(wg, a.ntiles_m, total, a.causal, bh, tile_m);
+    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // the last query tile sees the most keys
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
     const int query = m0 + 32 * wave + c; // this lane's query

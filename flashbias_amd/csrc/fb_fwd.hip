@@ -249,10 +249,9 @@ __device__ __forceinline__ void fwd_body(const FwdArgs &a) {
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_m * a.B * a.H;
-    const int work = xcd_remap(blockIdx.x, total);
-    const int bh = work / a.ntiles_m;
-    int tile_m = work % a.ntiles_m;
-    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // long rows first
+    int bh, tile_m;
+    work_order(blockIdx.x, a.ntiles_m, total, a.causal, bh, tile_m);
+    if (a.causal) tile_m = a.ntiles_m - 1 - tile_m; // the last query tile sees the most keys
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
     const int wq0 = m0 + wave * (32 * C::QB); // first query of this wave
@@ -552,16 +551,17 @@ static hipError_t launch_fwd_qb(const FwdArgs &a0, hipStream_t stream) {
 
 // Two query blocks per wave (256 queries per workgroup) pay once every compute unit has two such
 // workgroups; below that, 128-query workgroups at three waves per SIMD fill the chip better
-// (measured: 35 % faster at a quarter of that grid, 10 % slower at twice it).  Under a causal mask
-// the workgroups differ in length and the short ones leave the chip part empty towards the end:
-// the small workgroups stay ahead up to seven per compute unit (B1 H50 d32: 13 % faster at
-// L=4096, 5 % at L=8192, equal at L=16384).  Short sequences whose last 256-query workgroup would be half
+// (measured: 35 % faster at a quarter of that grid, 10 % slower at twice it).  Under a causal mask the
+// workgroups differ in length; with every XCD's share started longest first (work_order, fb_order.h) three
+// per compute unit are enough (B1 H50 d32 r16: 0.453 -> 0.434 ms at L=8192, 0.127 -> 0.125 at L=4096; while the
+// grid was walked head by head the small workgroups stayed ahead up to seven per compute unit).
+// Short sequences whose last 256-query workgroup would be half
 // empty also take the small ones (8192 x 16 windows of 128 tokens: 1.94 -> 1.41 ms).
 template <class T, int NKD, int NKR, int NDV, bool VEC, bool MASK, bool FOLD = false>
 static hipError_t launch_fwd_vec(const FwdArgs &a, hipStream_t stream) {
     if constexpr (FwdCfg<T, NKD, NKR, NDV, VEC, MASK, true>::QB == 2) {
         const int64_t wgs = (int64_t)a.B * a.H * ((a.Lq + 255) / 256);
-        if (wgs < (int64_t)(a.causal ? 7 : 2) * num_cus() || half_empty_256(a.Lq))
+        if (wgs < (int64_t)(a.causal ? 3 : 2) * num_cus() || half_empty_256(a.Lq))
             return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, false, FOLD>(a, stream);
     }
     return launch_fwd_qb<T, NKD, NKR, NDV, VEC, MASK, true, FOLD>(a, stream);

@@ -1,10 +1,32 @@
 // Sanitizer driver for the argument checks and size queries of the C ABI (fb_checks.cpp), built
 // under AddressSanitizer and UBSan by `make sanitize` and called with well-formed and with
-// deliberately malformed parameter blocks.  No GPU is involved.  Exit status 0 = clean.
+// deliberately malformed parameter blocks, and for the launch order of the kernels (fb_order.h).  No GPU is
+// involved.  Exit status 0 = clean.
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
+#include "fb_order.h"
 #include "flashbias.h"
+
+// Every (unit, position) pair exactly once; under a causal mask every XCD's share longest first.
+static bool launch_order_ok(int units, int ntiles, bool causal) {
+    const int total = units * ntiles;
+    std::vector<int> seen(total, 0);
+    std::vector<int> last(8, 0); // the position of the previous workgroup of each XCD's sequence
+    for (int wg = 0; wg < total; ++wg) {
+        int unit = -1, pos = -1;
+        fb::work_order(wg, ntiles, total, causal, unit, pos);
+        if (unit < 0 || unit >= units || pos < 0 || pos >= ntiles) return false;
+        if (seen[unit * ntiles + pos]++) return false;
+        if (causal) {
+            int &prev = last[total % 8 == 0 ? wg % 8 : 0];
+            if (pos < prev) return false;
+            prev = pos;
+        }
+    }
+    return true;
+}
 
 static fb_params good(int pass) {
     alignas(16) static char buf[64]; // (never dereferenced by the checks)
@@ -56,6 +78,13 @@ int main() {
     if (fb_bwd_workspace_bytes(&p) != (size_t)2 * 4 * 128 * (2 * sizeof(float) + 16)) bad = 1; // per query row: two floats, one chunk
     p.B = 0;
     if (fb_bwd_workspace_bytes(&p) != 0 || fb_bwd_workspace_bytes(nullptr) != 0) bad = 1;
+    for (int units : {1, 2, 3, 7, 8, 9, 16, 50, 64})
+        for (int ntiles : {1, 2, 3, 5, 8, 16, 31, 32, 64, 100, 128})
+            for (int causal = 0; causal < 2; ++causal)
+                if (!launch_order_ok(units, ntiles, causal != 0)) {
+                    std::fprintf(stderr, "launch order: %d units x %d tiles, causal %d\n", units, ntiles, causal);
+                    bad = 1;
+                }
     if (!bad) std::puts("sanitize_check: clean");
     return bad;
 }
