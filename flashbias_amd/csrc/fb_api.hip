@@ -20,6 +20,8 @@ FB_DECL(f16_1) FB_DECL(f16_2) FB_DECL(f16_4) FB_DECL(f16_8)
 #undef FB_DECL
 hipError_t launch_bwd_both_bf16_2(const BwdArgs &a, hipStream_t stream);
 hipError_t launch_bwd_both_f16_2(const BwdArgs &a, hipStream_t stream);
+hipError_t launch_bwd_both_general_bf16_2(const BwdArgs &a, hipStream_t stream);
+hipError_t launch_bwd_both_general_f16_2(const BwdArgs &a, hipStream_t stream);
 hipError_t launch_bwd_win_bf16_2(const BwdArgs &a, hipStream_t stream);
 hipError_t launch_bwd_win_f16_2(const BwdArgs &a, hipStream_t stream);
 
@@ -52,6 +54,10 @@ hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream) {
 // dq and dk/dv workgroups of the streamlined kernels in one launch (fb_bwd_both.hip; head dim 32)
 hipError_t launch_bwd_both(const BwdArgs &a, bool bf16, hipStream_t stream) {
     return bf16 ? launch_bwd_both_bf16_2(a, stream) : launch_bwd_both_f16_2(a, stream);
+}
+// the same for the general kernels with factors of rank 8 ... 32
+hipError_t launch_bwd_both_general(const BwdArgs &a, bool bf16, hipStream_t stream) {
+    return bf16 ? launch_bwd_both_general_bf16_2(a, stream) : launch_bwd_both_general_f16_2(a, stream);
 }
 // all five gradients of a short sequence in one workgroup (fb_bwd_win.hip; head dim 32)
 hipError_t launch_bwd_win(const BwdArgs &a, bool bf16, hipStream_t stream) {
@@ -252,13 +258,15 @@ int fb_bwd(const fb_params *p, void *stream) {
     fb::BwdArgs a = bwd_args(p);
     if (fb::window_backward(a)) // whole sequences of at most 256 positions: one workgroup per (batch, head), one launch
         return launched(fb::launch_bwd_win(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd (window)");
-    if (fb::mixed_backward(a)) {
+    const bool general_mix = p->dtype == FB_BF16 ? fb::mixed_general_backward<fb::BF16>(a) : fb::mixed_general_backward<fb::F16>(a);
+    if (fb::mixed_backward(a) || general_mix) {
         // small grids of the streamlined kernels: the preprocess step, then one launch that holds the dq and
         // the dk/dv workgroups side by side (same bits as the two launches)
         const int rc1 = launched(fb::launch_bwd_preprocess(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
                                  "fb_bwd_preprocess");
         if (rc1) return rc1;
-        return launched(fb::launch_bwd_both(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd (dq + dk/dv)");
+        return launched((general_mix ? fb::launch_bwd_both_general : fb::launch_bwd_both)(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)),
+                        "fb_bwd (dq + dk/dv)");
     }
     a.stats_here = 1;
     const int rc2 = launched(fb::launch_bwd_dq(a, p->dtype == FB_BF16, static_cast<hipStream_t>(stream)), "fb_bwd_dq");

@@ -114,6 +114,15 @@ inline bool mixed_backward(const BwdArgs &a0) {
     return ndq % 8 == 0 && ndkv % 8 == 0 && ndq <= num_cus() && ndkv <= num_cus();
 }
 
+// The same question for the general dq and dk/dv kernels of head dim 32 with factors (launch_both_general in
+// fb_bwd_both.hip): both kernels would run their aligned, unmasked 128-row instantiations with the same folding of
+// the scale, the counts of both kinds split evenly over the eight XCDs, and the grid is small: at most one
+// workgroup per compute unit and kind, or, under a causal mask, at most one and a half per workgroup slot (three
+// slots per compute unit), where a launch's length is that of its longest workgroup and the two kinds fill each
+// other's tails.  Declared after fold_scale_ok below.
+template <class T>
+inline bool mixed_general_backward(const BwdArgs &a0);
+
 // Whether fb_bwd runs the window kernel (fb_bwd_win.hip: one workgroup per (batch, head) forms the per-query
 // statistics and all five gradients, dq summed inside the workgroup) instead of the dq and dk/dv launches: whole
 // sequences of at most 256 positions, head dim 32, rank a multiple of 8 up to 32, aligned tensors, no additive or
@@ -196,6 +205,24 @@ inline bool fold_scale_ok(float scale, int r, int len) {
     if (!T::kWideRange || len < 512) return false;
     int e;
     return r <= 8 || std::frexp(scale, &e) == 0.5f;
+}
+
+template <class T>
+inline bool mixed_general_backward(const BwdArgs &a0) {
+    BwdArgs a = a0;
+    a.stats_here = 0;
+    const int64_t lim = (int64_t)1 << 24;
+    if (!(a.d == 32 && a.r >= 8 && a.r <= 32 && a.r % 8 == 0 && a.mask.type == 0) || dq_streamlined(a) || dkv_streamlined(a)) return false;
+    if (!(a.q.vec_ok && a.k.vec_ok && a.v.vec_ok && a.dout.vec_ok && a.qb.vec_ok && a.kb.vec_ok && a.q.ss < lim && a.k.ss < lim &&
+          a.v.ss < lim && a.dout.ss < lim && a.qb.ss < lim && a.kb.ss < lim))
+        return false;
+    if (fold_scale_ok<T>(a.scale, a.r, a.Lk) != fold_scale_ok<T>(a.scale, a.r, a.Lq)) return false;
+    const int group = a.group > 1 ? a.group : 1;
+    const int64_t units = (int64_t)((a.B + group - 1) / group) * a.H;
+    const int64_t ndq = units * ((a.Lq + 127) / 128), ndkv = units * ((a.Lk + 127) / 128);
+    if (ndq % 8 != 0 || ndkv % 8 != 0) return false;
+    const int64_t most = ndq > ndkv ? ndq : ndkv;
+    return most <= num_cus() || (a.causal && 2 * most <= 9 * (int64_t)num_cus());
 }
 
 } // namespace fb

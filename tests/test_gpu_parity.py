@@ -463,9 +463,13 @@ def test_backward_phases_through_the_c_abi(gpu_device):
     (torch.bfloat16, 2, 4, 1024, 1024, 8, False), (torch.float16, 2, 4, 2048, 2048, 8, True),
     (torch.bfloat16, 2, 4, 4096, 4096, 0, False), (torch.bfloat16, 1, 8, 1000, 3000, 8, False),
     (torch.bfloat16, 4, 2, 2500, 1111, 8, True), (torch.float16, 2, 4, 1100, 1100, 8, False),
-    (torch.bfloat16, 1, 4, 640, 700, 0, False)])
+    (torch.bfloat16, 1, 4, 640, 700, 0, False),
+    # the general kernels (ranks 16 ... 32): small grids, and causal grids of up to 1.5 workgroups per slot and kind
+    (torch.bfloat16, 1, 48, 2048, 2048, 16, True), (torch.float16, 2, 4, 1024, 1024, 16, False),
+    (torch.bfloat16, 2, 8, 700, 1500, 32, True), (torch.float16, 1, 8, 1024, 1000, 24, False)])
 def test_small_grid_backward_in_one_launch(gpu_device, dtype, B, H, Lq, Lk, r, causal):
-    """On grids that give neither backward kernel more than one workgroup per compute unit fb_bwd runs
+    """On grids that give neither backward kernel more than one workgroup per compute unit (with factors of rank 16
+    and more under a causal mask: up to one and a half per workgroup slot) fb_bwd runs
     the preprocess step and one launch that holds the dq and the dk/dv workgroups side by side: the
     gradients and the scratch buffer are bit for bit those of the three phases launched one by one,
     and the gradients pass the gate against the oracle (ragged and rectangular shapes, even and odd
@@ -501,7 +505,10 @@ def test_small_grid_backward_in_one_launch(gpu_device, dtype, B, H, Lq, Lk, r, c
         _lib.check_status(getattr(lib, name)(p2, _stream()))
     torch.cuda.synchronize()
     for name in whole:
-        assert torch.equal(whole[name], parts[name]), name
+        if name == "scratch":  # (bit patterns: what neither path writes is still the NaN it was filled with)
+            assert torch.equal(whole[name].view(torch.int32), parts[name].view(torch.int32)), name
+        else:
+            assert torch.equal(whole[name], parts[name]), name
     ref = oracle(q, k, v, qb, kb, None, causal, None, do)
     cpu = lambda t: t.detach().float().cpu()
     assert (cpu(whole["o"]) - ref[0]).abs().max() <= O_TOL[dtype]
