@@ -14,7 +14,7 @@ FB_MASK_NONE, FB_MASK_VECTOR, FB_MASK_MATRIX = 0, 1, 2
 
 #: every symbol that include/flashbias.h declares
 EXPORTS = ("fb_version", "fb_init", "fb_last_error", "fb_bwd_workspace_bytes", "fb_suggest_bias_grad_group", "fb_check", "fb_fwd", "fb_bwd",
-           "fb_sum_over_batch",
+           "fb_sum_over_batch", "fb_resize_rank",
            "fb_bwd_preprocess", "fb_bwd_dkv", "fb_bwd_dq", "fb_bwd_static")
 
 
@@ -74,6 +74,8 @@ def load():
     lib.fb_sum_over_batch.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int64,
                                       ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p]
     lib.fb_sum_over_batch.restype = ctypes.c_int
+    lib.fb_resize_rank.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.fb_resize_rank.restype = ctypes.c_int
     _lib = lib
     return lib
 

@@ -231,6 +231,14 @@ int fb_sum_over_batch(const void *full, void *out, int dtype, int out_dtype, int
                     "fb_sum_over_batch");
 }
 
+int fb_resize_rank(const void *in, void *out, int64_t rows, int r_in, int r_out, void *stream) {
+    fb::api_clear_error();
+    if (!in || !out) return fb::api_fail(FB_ERR_NULL, "fb_resize_rank: null pointer");
+    if (rows <= 0 || r_in <= 0 || r_out <= 0 || r_in > 4096 || r_out > 4096 || (rows + 255) / 256 > 0x7fffffff)
+        return fb::api_fail(FB_ERR_SHAPE, "fb_resize_rank: rows and both ranks must be positive (ranks up to 4096, rows below 2^39)");
+    return launched(fb::launch_resize_rank(in, out, rows, r_in, r_out, static_cast<hipStream_t>(stream)), "fb_resize_rank");
+}
+
 int fb_bwd_static(const fb_params *p, void *stream) {
     // fb_bwd with the scratch buffer taken from the library's own static device array instead of
     // fb_params.delta (which is ignored): no allocation, here or in anything it calls.

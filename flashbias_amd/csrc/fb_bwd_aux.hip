@@ -174,6 +174,35 @@ hipError_t launch_sum_over_batch(const void *full, void *out, bool bf16, bool ou
     return hipGetLastError();
 }
 
+// out[row][c] = c < min(r_in, r_out) ? in[row][c] : 0 for contiguous rows of 16-bit elements: one thread per row.
+__global__ __launch_bounds__(256) void resize_rank_kernel(const uint16_t *in, uint16_t *out, int64_t rows, int r_in, int r_out) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (row >= rows) return;
+    const uint16_t *src = in + row * r_in;
+    uint16_t *dst = out + row * r_out;
+    const int keep = r_in < r_out ? r_in : r_out;
+    if (r_out % 8 == 0 && keep <= 8 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+        // the usual case (a rank below 8 padded to 8 or 16): the row leaves as 16-byte stores
+        uint16_t x[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) x[c] = c < keep ? src[c] : (uint16_t)0;
+        u32x4_t first;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) first[e] = (uint32_t)x[2 * e] | ((uint32_t)x[2 * e + 1] << 16);
+        *reinterpret_cast<u32x4_t *>(dst) = first;
+        for (int c = 8; c < r_out; c += 8) *reinterpret_cast<u32x4_t *>(dst + c) = u32x4_t{0u, 0u, 0u, 0u};
+        return;
+    }
+    for (int c = 0; c < r_out; ++c) dst[c] = c < keep ? src[c] : (uint16_t)0;
+}
+
+hipError_t launch_resize_rank(const void *in, void *out, int64_t rows, int r_in, int r_out, hipStream_t stream) {
+    (void)hipGetLastError();
+    hipLaunchKernelGGL(resize_rank_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<const uint16_t *>(in), static_cast<uint16_t *>(out), rows, r_in, r_out);
+    return hipGetLastError();
+}
+
 hipError_t launch_bwd_preprocess(const BwdArgs &a, bool bf16, hipStream_t stream) {
     (void)hipGetLastError(); // (an earlier, unrelated error of the process is not this launch's)
     if (bf16)

@@ -48,6 +48,9 @@ hipError_t launch_bwd_dq(const BwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_sum_over_batch(const void *full, void *out, bool bf16, bool out_f32, int64_t B, int64_t n, int64_t sb,
                                  hipStream_t stream);
 
+// out[row][c] = c < min(r_in, r_out) ? in[row][c] : 0: contiguous rows of 16-bit elements.
+hipError_t launch_resize_rank(const void *in, void *out, int64_t rows, int r_in, int r_out, hipStream_t stream);
+
 // Compute units of the current device (cached per device; 256 on MI355X).  The launchers pick
 // smaller query tiles when the larger ones would leave compute units without a workgroup.
 inline int num_cus() {

@@ -192,6 +192,29 @@ struct FlashBiasFn : public torch::autograd::Function<FlashBiasFn> {
     }
 };
 
+// x (..., r) with its last dim zero-padded (or cut) to `rank` columns in one launch of the library; the gradient
+// is the same operation the other way.  For contiguous 16-bit GPU tensors (the caller checks).
+struct ResizeRankFn : public torch::autograd::Function<ResizeRankFn> {
+    static Tensor forward(AutogradContext *ctx, const Tensor &x, int64_t rank) {
+        TORCH_CHECK(x.is_cuda() && x.is_contiguous() && x.element_size() == 2 && x.dim() >= 1 && x.numel() > 0 && rank > 0,
+                    "resize_rank wants a contiguous fp16 / bf16 GPU tensor");
+        ctx->saved_data["rank_in"] = x.size(-1);
+        auto shape = x.sizes().vec();
+        shape.back() = rank;
+        Tensor out = torch::empty(shape, x.options());
+        const c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+        check(fb_resize_rank(x.data_ptr(), out.data_ptr(), out.numel() / rank, (int)x.size(-1), (int)rank,
+                             c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(x.device().index()).stream()));
+        return out;
+    }
+
+    static tensor_list backward(AutogradContext *ctx, tensor_list grads) {
+        return {ResizeRankFn::apply(grads[0].contiguous(), ctx->saved_data["rank_in"].toInt()), Tensor()};
+    }
+};
+
+Tensor resize_rank(const Tensor &x, int64_t rank) { return ResizeRankFn::apply(x, rank); }
+
 Tensor flash_bias(const Tensor &q, const Tensor &k, const Tensor &v, const c10::optional<Tensor> &q_bias,
                   const c10::optional<Tensor> &k_bias, const c10::optional<Tensor> &mask, bool causal, double softmax_scale) {
     return FlashBiasFn::apply(q, k, v, q_bias, k_bias, mask, causal, softmax_scale);
@@ -203,6 +226,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.doc() = "flash_bias_func with its autograd function in C++ (kernel-ready inputs; see flashbias_amd/interface.py)";
     // what this module was compiled against: the caller compares both with the library it loaded
     m.def("abi", []() { return std::make_pair((int)FB_VERSION, (int)sizeof(fb_params)); });
+    m.def("resize_rank", &resize_rank, py::arg("x"), py::arg("rank"));
     m.def("flash_bias", &flash_bias, py::arg("q"), py::arg("k"), py::arg("v"), py::arg("q_bias") = py::none(),
           py::arg("k_bias") = py::none(), py::arg("mask") = py::none(), py::arg("causal") = false,
           py::arg("softmax_scale") = 0.0);

@@ -70,6 +70,16 @@ def _fold_vector_mask(q, q_bias, k_bias, mask):
     return q_new, k_new
 
 
+def _resize_rank(x, rank):
+    """`x` (..., r) with its last dim zero-padded to `rank`: one launch of the library (fb_resize_rank, through the
+    C++ extension's autograd function) for contiguous 16-bit GPU tensors, the tensor library's pad otherwise (a
+    permuted view keeps its permuted layout there)."""
+    ext = _extension()
+    if ext is not None and x.is_cuda and x.is_contiguous() and x.element_size() == 2 and x.numel() > 0:
+        return ext.resize_rank(x, rank)
+    return torch.nn.functional.pad(x, (0, rank - x.shape[-1]))
+
+
 def _prepare_factors(q, k, q_bias, k_bias, mask):
     """What the kernels get in place of (q_bias, k_bias, mask): a large vector mask folded into the
     factors, the rank zero-padded to a multiple of 8, the channel dimension contiguous.  Done once
@@ -99,8 +109,7 @@ def _prepare_factors(q, k, q_bias, k_bias, mask):
             # over points in a unit box) opts in to rank 8 by padding them itself, once
             # (factors.pad_rank): the choice depends on nothing but the shapes it passes.
             target = 16 if rank < 8 else -(-rank // 8) * 8
-            pad = (0, target - rank)
-            q_bias, k_bias = torch.nn.functional.pad(q_bias, pad), torch.nn.functional.pad(k_bias, pad)
+            q_bias, k_bias = _resize_rank(q_bias, target), _resize_rank(k_bias, target)
         # (padding a permuted view keeps its permuted layout)
         q_bias, k_bias = _last_dim_contiguous(q_bias), _last_dim_contiguous(k_bias)
     if mask is not None:

@@ -178,6 +178,14 @@ int fb_bwd_static(const fb_params *p, void *stream);
 int fb_sum_over_batch(const void *full, void *out, int dtype, int out_dtype, int64_t B, int64_t n,
                       int64_t batch_stride, void *stream);
 
+/* Factors of a rank that is no multiple of 8 (ALiBi: 2, a distance bias in three dimensions: 5) have rows the
+ * kernels' 16-byte loads cannot take; their owner, or the operator on every call, pads them with zero columns,
+ * which change nothing in q_bias k_bias^T.  out[row][c] = c < min(r_in, r_out) ? in[row][c] : 0 for `rows`
+ * contiguous rows of 16-bit elements (either dtype): r_out > r_in pads, r_out < r_in takes the original columns of
+ * a gradient back out.  One launch.  The reference pads inside its kernels instead (BLOCK_RANKDIM, the next power
+ * of two of at least 16, with masked loads: flash_bias_triton.py:1137, :195-200). */
+int fb_resize_rank(const void *in, void *out, int64_t rows, int r_in, int r_out, void *stream);
+
 /* The backward in three phases, exported so that a harness can time them separately (call them in
  * this order: the two main kernels read what the preprocess wrote).
  *   fb_bwd_preprocess: delta = rowsum(o * dout)       (_bwd_preprocess_do_o_dot, :358-400); fills the

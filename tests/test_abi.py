@@ -170,6 +170,16 @@ def test_sum_over_batch_rejects(args, code):
     assert lib.fb_last_error() != b""
 
 
+@pytest.mark.parametrize("args,code", [
+    ((None, 0x2000, 10, 2, 16), -1), ((0x1000, None, 10, 2, 16), -1),
+    ((0x1000, 0x2000, 0, 2, 16), -2), ((0x1000, 0x2000, 10, 0, 16), -2), ((0x1000, 0x2000, 10, 2, 5000), -2),
+])
+def test_resize_rank_rejects(args, code):
+    lib = _lib.load()
+    assert lib.fb_resize_rank(*args, None) == code  # rejected before any launch
+    assert lib.fb_last_error() != b""
+
+
 def test_null_params():
     lib = _lib.load()
     assert lib.fb_check(None, 0) == -1

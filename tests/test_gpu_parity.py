@@ -648,6 +648,47 @@ def test_window_backward(gpu_device, dtype, B, H, Lq, Lk, r, scale, group, grads
             assert errors(got, want)[1] <= max(tol, GRAD_TOL), name
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,r_in,r_out", [(1000, 2, 16), (777, 5, 8), (300, 7, 16), (513, 16, 2), (129, 8, 5), (64, 20, 24),
+                                             (50, 3, 6), (1, 1, 8)])
+def test_resize_rank(gpu_device, dtype, rows, r_in, r_out):
+    """fb_resize_rank through the C ABI: zero columns appended, or the first columns taken, bit for bit; also
+    into an output that is not 16-byte aligned."""
+    from flashbias_amd import _lib
+    from flashbias_amd.interface import _stream
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(rows, r_in, generator=g).to(dtype).to(gpu_device)
+    keep = min(r_in, r_out)
+    want = torch.zeros(rows, r_out, dtype=dtype, device=gpu_device)
+    want[:, :keep] = x[:, :keep]
+    for offset in (0, 1):
+        buf = torch.full((rows * r_out + 8,), float("nan"), dtype=dtype, device=gpu_device)
+        out = buf[offset:offset + rows * r_out].view(rows, r_out)
+        _lib.check_status(lib.fb_resize_rank(x.data_ptr(), out.data_ptr(), rows, r_in, r_out, _stream()))
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
+        assert torch.isnan(buf[offset + rows * r_out:].float()).all() and torch.isnan(buf[:offset].float()).all()
+
+
+def test_rank_padding_inside_the_operator(gpu_device):
+    """Factors of rank 5 through flash_bias_func (padded per call by the library's kernel, their gradients cut
+    back by it) against the same factors padded by the tensor library beforehand: same bits."""
+    B, L, H, d, r = 2, 300, 3, 32, 5
+    q, k, v, qb, kb, do = [t.to(gpu_device) for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=51)]
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, qb, kb)]
+    got = torch.autograd.grad(flash_bias_func(*leaves, None, True, None), leaves, do)
+    leaves2 = [t.clone().requires_grad_(True) for t in (q, k, v, qb, kb)]
+    pad = lambda t: torch.nn.functional.pad(t, (0, 16 - r))  # (ranks below 8 go to 16)
+    want = torch.autograd.grad(flash_bias_func(*leaves2[:3], pad(leaves2[3]), pad(leaves2[4]), None, True, None), leaves2, do)
+    for a, b in zip(got, want):
+        assert a.shape == b.shape and torch.equal(a, b)
+    # a permuted view (what the reference's harness passes, benchmark.py:233-235) takes the tensor library's pad
+    qbp = qb.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3).requires_grad_(True)
+    got2 = torch.autograd.grad(flash_bias_func(leaves[0], leaves[1], leaves[2], qbp, leaves[4], None, True, None), [qbp], do)
+    assert torch.equal(got2[0], got[3])
+
+
 def _random_windows(count, seed):
     """Reproducible draws from what the window backward accepts: any lengths up to 256, ranks 0 ... 32 in steps of
     8, both element types, factors per entry or shared with groups of any size, with or without factor gradients,
