@@ -265,6 +265,25 @@ def _device_configs(dev):
     return cfgs
 
 
+def _swin_accuracy(dev):
+    """What configuration 4 asks to be reported beside its timings: how well the rank-16 factors reproduce the
+    bias table (relative Frobenius error, worst head) and how far the operator's output is from the attention
+    with the dense table and from the oracle on the same factors (eight windows, fp32 oracle on the CPU)."""
+    import torch
+    from flashbias_amd import flash_bias_func, workloads
+    from oracle import eager
+    w = workloads.swin(windows=8)
+    with torch.no_grad():
+        o = flash_bias_func(*(w[n].to(dev) for n in ("q", "k", "v", "q_bias", "k_bias")), None, False,
+                            w["softmax_scale"]).float().cpu()
+    f = lambda n: w[n].float()
+    dense = eager.attention_eager(f("q"), f("k"), f("v"), w["softmax_scale"], w["bias_table"][None].expand(8, -1, -1, -1))
+    same = eager.flashbias_eager(f("q"), f("k"), f("v"), f("q_bias"), f("k_bias"), None, False, w["softmax_scale"])
+    return {"bias_reconstruction_rel_error": round(float(w["bias_rel_error"].max()), 5),
+            "o_max_abs_err_vs_dense_table": round(float((o - dense).abs().max()), 5),
+            "o_max_abs_err_vs_oracle_on_the_factors": round(float((o - same).abs().max()), 5)}
+
+
 def _sweep(dev, steps, warmup, only=None):
     import torch
     from flashbias_amd import workloads
@@ -297,6 +316,8 @@ def _sweep(dev, steps, warmup, only=None):
                     "pct_of_hbm_peak": round(100 * hbm / t_fb / 1e6 / PEAK_HBM_GBS, 2)})
         del q, k, v, qb, kb, do, leaves
         torch.cuda.empty_cache()
+        if name.startswith("swin"):
+            out[-1].update(_swin_accuracy(dev))
     return out
 
 
