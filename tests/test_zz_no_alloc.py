@@ -49,9 +49,10 @@ def test_static_scratch_backward_matches_fb_bwd(gpu_device):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("dtype,B,L,H,causal", [(torch.float16, 2, 1024, 4, False),   # small grid: preprocess + one mixed launch
-                                                (torch.bfloat16, 3, 520, 8, True)])
-def test_static_scratch_backward_in_a_graph(gpu_device, dtype, B, L, H, causal):
+@pytest.mark.parametrize("dtype,B,L,H,causal,r", [(torch.float16, 2, 1024, 4, False, 8),   # small grid: preprocess + one mixed launch
+                                                  (torch.bfloat16, 3, 520, 8, True, 8),
+                                                  (torch.bfloat16, 2, 640, 8, True, 16)])   # ... of the general kernels
+def test_static_scratch_backward_in_a_graph(gpu_device, dtype, B, L, H, causal, r):
     """fb_bwd_static captured in a HIP graph after fb_init() (the address of the static array is looked up outside
     the capture) and replayed three times with the program's own eager work between the replays: every replay's
     gradients are bit for bit those of fb_bwd."""
@@ -60,7 +61,7 @@ def test_static_scratch_backward_in_a_graph(gpu_device, dtype, B, L, H, causal):
     dev = gpu_device
     lib = _lib.load()
     assert lib.fb_init() == 0
-    q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, 32, 8, dtype, seed=23)]
+    q, k, v, qb, kb, do = [t.to(dev) for t in make_inputs(B, L, L, H, 32, r, dtype, seed=23)]
     p, keep = _params(q, k, v, qb, kb, None, causal, None)
     o, lse = torch.empty_like(q), torch.empty((B, H, L), device=dev, dtype=torch.float32)
     names = ("dq", "dk", "dv", "dqb", "dkb")
