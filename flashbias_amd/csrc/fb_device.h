@@ -425,9 +425,9 @@ __device__ __forceinline__ void mask_block_queries(const MaskDesc &m, const uint
 // consecutive ids to the 8 XCDs round-robin) cover a contiguous range of logical ids and so
 // share K/V of the same (batch, head) in that XCD's L2.
 __device__ __forceinline__ int xcd_remap(int wg, int total) {
-    constexpr int kXcd = 8;
-    if (total % kXcd != 0) return wg;
-    return (wg % kXcd) * (total / kXcd) + wg / kXcd;
+    int work, none;
+    work_order(wg, 1, total, false, work, none); // (fb_order.h: the shares of any total, walked in order)
+    return work;
 }
 
 // max(x of this lane, x of lane ^ 32): v_permlane32_swap exchanges the upper half of its first

@@ -13,7 +13,7 @@ namespace fb {
 // Workgroup `wg` of a launch of `total` = units x ntiles workgroups takes tile `pos` of unit `unit`.  The hardware
 // deals workgroup ids round-robin over the 8 XCDs and starts them in the order of their ids.  Each XCD gets one
 // contiguous share of the unit-major numbering (unit * ntiles + pos), so that the workgroups of a unit meet in one
-// L2 (when the total does not divide by 8 there is one share for all).  Without a causal mask the share is walked
+// L2.  Without a causal mask the share is walked
 // in that numbering.  Under a causal mask `pos` counts a unit's tiles from the longest, a workgroup's length falls
 // from ntiles to 1 key (query) tiles, and walking unit by unit ends every share with the long workgroups of its
 // last unit while most of the chip has run dry (B1 H50 L=4096 in 128-row tiles: 60 tile times for a share of 200
@@ -22,13 +22,9 @@ namespace fb {
 // each other and sweep the keys together.
 FB_HD void work_order(int wg, int ntiles, int total, bool causal, int &unit, int &pos) {
     constexpr int kXcd = 8;
-    int w0 = 0, w1 = total, j = wg;
-    if (total % kXcd == 0) {
-        const int per = total / kXcd;
-        w0 = (wg % kXcd) * per;
-        w1 = w0 + per;
-        j = wg / kXcd;
-    }
+    // XCD x receives the ids x, x + 8, ...: total / 8 of them, one more on the first total % 8 XCDs
+    const int x = wg % kXcd, j = wg / kXcd, per = total / kXcd, more = total % kXcd;
+    const int w0 = x * per + (x < more ? x : more), w1 = w0 + per + (x < more ? 1 : 0);
     const int ua = w0 / ntiles, p0 = w0 % ntiles; // the share's first unit, from position p0 on
     if (!causal) {
         unit = (w0 + j) / ntiles;

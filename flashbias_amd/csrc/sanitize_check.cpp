@@ -14,18 +14,24 @@ static bool launch_order_ok(int units, int ntiles, bool causal) {
     const int total = units * ntiles;
     std::vector<int> seen(total, 0);
     std::vector<int> last(8, 0); // the position of the previous workgroup of each XCD's sequence
+    std::vector<int> lo(8, total), hi(8, -1); // the range of the unit-major numbering each XCD serves
     for (int wg = 0; wg < total; ++wg) {
         int unit = -1, pos = -1;
         fb::work_order(wg, ntiles, total, causal, unit, pos);
         if (unit < 0 || unit >= units || pos < 0 || pos >= ntiles) return false;
         if (seen[unit * ntiles + pos]++) return false;
+        if (unit * ntiles + pos < lo[wg % 8]) lo[wg % 8] = unit * ntiles + pos;
+        if (unit * ntiles + pos > hi[wg % 8]) hi[wg % 8] = unit * ntiles + pos;
         if (causal) {
-            int &prev = last[total % 8 == 0 ? wg % 8 : 0];
+            int &prev = last[wg % 8];
             if (pos < prev) return false;
             prev = pos;
         }
     }
-    return true;
+    int count = 0; // the shares are contiguous: their extents add up to the total
+    for (int x = 0; x < 8; ++x)
+        if (hi[x] >= 0) count += hi[x] - lo[x] + 1;
+    return count == total;
 }
 
 static fb_params good(int pass) {
