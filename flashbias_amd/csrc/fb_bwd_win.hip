@@ -59,7 +59,11 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    const int group = a.group > 1 ? a.group : 1;
+    // A workgroup walks `group` consecutive batch entries (the next one's tiles travel while this one computes).
+    // With a.group > 1 their factor gradients are summed into row bg of the gradient tensors; otherwise the walk
+    // is the launcher's choice (a.walk) and every entry's factor gradients are stored as its own rows.
+    const bool summed = a.group > 1;
+    const int group = summed ? a.group : (a.walk > 1 ? a.walk : 1);
     const int nbg = (a.B + group - 1) / group;
     const int work = xcd_remap(blockIdx.x, nbg * a.H);
     const int bg = work / a.H, h = work % a.H;
@@ -161,6 +165,19 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 #pragma unroll
         for (int j = 0; j < 2; ++j) so[j] = *reinterpret_cast<const u32x4_t *>(orow + 8 * j);
         slse = a.lse[((int64_t)b * a.H + h) * a.Lq + rr];
+    };
+    // dk_bias (one accumulator block per wave, its keys) and dq_bias (one block per wave: queries
+    // 128 (wave / 4) + 32 (wave % 4) ..) into row `row_b` of the gradient tensors
+    auto factor_gradients = [&](int row_b) {
+        if constexpr (C::BG) {
+            const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+            const int c = lane_end & 31, g = lane_end >> 5;
+            dkv_store<T, C, true>(a, acc_dv, acc_dk, row_b, h, wk0, c, g);
+            const int query = C::BMQ * (wave >> 2) + 32 * nb + c;
+            const bool ok = query < a.Lq;
+            uint16_t *row = const_cast<uint16_t *>(a.dqb.ptr) + row_b * a.dqb.sb + h * a.dqb.sh + (int64_t)(ok ? query : 0) * a.dqb.ss;
+            store_acc_rows<T, true>(row, ok, a.dqb.vec_ok, acc_dqb, 1.f, a.r, g);
+        }
     };
     if (bg * group < a.B) { // the first window of the workgroup: everything at once
         const int b0 = __builtin_amdgcn_readfirstlane(bg * group);
@@ -349,20 +366,22 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
             }
             barrier_lds(); // everyone has read the dS tile
         }
+        if constexpr (C::BG) {
+            if (!summed && a.dkb.ptr) { // this entry's own factor gradients; the accumulators start the next entry at zero
+                factor_gradients(b);
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    acc_dqb[v] = 0.f;
+#pragma unroll
+                    for (int n = 1; n < C::MB1; ++n) acc_dk[0][n][v] = 0.f;
+                }
+            }
+        }
     }
 
     // ---- the factor gradients, summed over the group's batch entries
     if constexpr (C::BG) {
-        if (a.dkb.ptr) {
-            const int lane_end = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-            const int c = lane_end & 31, g = lane_end >> 5;
-            dkv_store<T, C, true>(a, acc_dv, acc_dk, bg, h, wk0, c, g);
-            // this wave's dq_bias block: queries 128 (wave / 4) + 32 (wave % 4) ..
-            const int query = C::BMQ * (wave >> 2) + 32 * nb + c;
-            const bool ok = query < a.Lq;
-            uint16_t *row = const_cast<uint16_t *>(a.dqb.ptr) + bg * a.dqb.sb + h * a.dqb.sh + (int64_t)(ok ? query : 0) * a.dqb.ss;
-            store_acc_rows<T, true>(row, ok, a.dqb.vec_ok, acc_dqb, 1.f, a.r, g);
-        }
+        if (summed && a.dkb.ptr) factor_gradients(bg);
     }
 }
 
@@ -373,8 +392,16 @@ static hipError_t launch_win_cfg(const BwdArgs &a, hipStream_t stream) {
     static KernelOnce once;
     const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
     if (e != hipSuccess) return e;
-    const int group = a.group > 1 ? a.group : 1;
-    return launch_flat(kern, (int64_t)((a.B + group - 1) / group) * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
+    BwdArgs b = a;
+    b.walk = 1;
+    if (a.group <= 1) // nothing to sum: walk as many entries as leave four workgroups per compute unit
+        for (int w = 32; w > 1; w /= 2)
+            if ((int64_t)((a.B + w - 1) / w) * a.H >= 4 * (int64_t)num_cus()) {
+                b.walk = w;
+                break;
+            }
+    const int group = a.group > 1 ? a.group : b.walk;
+    return launch_flat(kern, (int64_t)((a.B + group - 1) / group) * a.H, C::NTHREADS, C::LDS_BYTES, stream, b);
 }
 
 template <class T, int NKR>

@@ -37,6 +37,7 @@ struct BwdArgs {
     int stats_here; // dq kernel: compute -delta and lse * log2(e) itself (and store them) instead of reading them
     int stat_chunks; // writers of the scratch buffer: also store the statistics chunks (dkv_streamlined())
     int group; // > 1: a workgroup serves this many consecutive batch entries and sums their factor gradients (row b / group)
+    int walk;  // window backward without such sums: batch entries a workgroup walks (set by its launcher)
 };
 
 // Each returns hipSuccess or the launch error.  `bf16` selects the element type.

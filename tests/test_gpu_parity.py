@@ -591,6 +591,10 @@ def test_factor_gradients_summed_over_batch_groups(gpu_device, dtype, B, Lq, Lk,
     (torch.float16, 256, 1, 129, 255, 0, None, 1, True),     # no factors
     (torch.bfloat16, 36, 8, 250, 250, 16, None, 1, False),   # constant factors: no dq_bias / dk_bias
     (torch.bfloat16, 64, 4, 256, 256, 8, None, 8, False),    # constant shared factors, groups
+    # enough (batch, head) pairs for a workgroup to walk several entries without summing their factor gradients
+    (torch.bfloat16, 1101, 4, 200, 256, 16, None, 1, True),  # four per workgroup, the last workgroup ragged
+    (torch.float16, 2100, 1, 129, 255, 0, None, 1, True),    # no factors, two per workgroup
+    (torch.bfloat16, 4100, 2, 64, 64, 8, 1.0, 1, False),     # constant factors, eight per workgroup
 ])
 def test_window_backward(gpu_device, dtype, B, H, Lq, Lk, r, scale, group, grads):
     """Whole sequences of at most 256 positions at head dim 32 on grids that fill the chip: fb_bwd runs the
