@@ -1,4 +1,4 @@
-"""The ctypes binding printed in INTEGRATION.md is executed as printed: its parameter block must be the
+"""The ctypes binding printed in the integration notes at the repository root is executed as printed: its parameter block must be the
 one the library expects (size check of every entry point, FB_ERR_ABI otherwise) and its field
 offsets those of flashbias_amd/_lib.py."""
 import ctypes
@@ -6,17 +6,18 @@ import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+NOTES = "INTEGRATION.md"
 
 
 def _documented_binding():
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(os.path.join(ROOT, NOTES)).read()
     blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
     block = next(b for b in blocks if "class FbParams" in b)
     ns = {}
     cwd = os.getcwd()
     os.chdir(ROOT)  # (the snippet loads the library by its path from the repository root)
     try:
-        exec(compile(block, "INTEGRATION.md", "exec"), ns)
+        exec(compile(block, NOTES, "exec"), ns)
     finally:
         os.chdir(cwd)
     return ns
@@ -48,6 +49,6 @@ def test_documented_parameter_block_is_accepted():
 
 def test_every_export_is_listed_in_the_document():
     from flashbias_amd import _lib
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(os.path.join(ROOT, NOTES)).read()
     for name in _lib.EXPORTS:
         assert name in text, name
