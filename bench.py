@@ -38,6 +38,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA
 PEAK_HBM_GBS = 8000.0
+MIN_WARM_SECONDS = 0.1  # of untimed calls before every event-timed measurement (_time_events)
 PROFILE_SUMMARY = os.path.join(ROOT, "profiles", "headline_fwd_bwd_kernels.md")
 
 
@@ -68,9 +69,15 @@ def _time_events(fn, steps, warmup, isolated=False):
     a kernel trace reports as a launch's duration); otherwise one pair around all the calls
     (throughput of back-to-back launches)."""
     import torch
+    t0 = time.perf_counter()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    # (whatever ran before may have left the GPU idle for a while, building inputs on the host for instance: at
+    # least a tenth of a second of calls before anything is timed)
+    while time.perf_counter() - t0 < MIN_WARM_SECONDS:
+        fn()
+        torch.cuda.synchronize()
     if isolated:
         pairs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
         for start, end in pairs:
