@@ -311,6 +311,7 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
     };
 
     int it = tile0, stg = 0; // stg: the stage of tile `it` (columns); the rows are one stage ahead
+    int turn = __builtin_amdgcn_readfirstlane(cu_slot());
     auto tile = [&](auto edge_tag) {
         constexpr bool EDGE = decltype(edge_tag)::value;
         const int m0 = it * C::BM;
@@ -318,6 +319,7 @@ __device__ __forceinline__ void bwd_dkv_lean_body(const BwdArgs &a, int wg, cons
         // has used what it read of tile it - 2
         wait_tiles(min(2, ntiles_m - 2 - it));
         asm volatile("s_barrier" ::: "memory");
+        take_turn(turn, a.slots); // (the two workgroups of a compute unit swap wave priority at every tile, as in the forward)
         if (it + C::NSTAGE - 2 < ntiles_m) issue(stg < 2 ? stg + C::NSTAGE - 2 : stg - 2, it + C::NSTAGE - 2);
         if (EDGE) hide(s0, m0);
         FB_SLOT_END;
@@ -374,7 +376,9 @@ static hipError_t launch_dkv_lean(const BwdArgs &a0, hipStream_t stream) {
     static KernelOnce once;
     const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
     if (e != hipSuccess) return e;
-    return launch_flat(kern, (int64_t)a.ntiles_n * a.B * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
+    const int64_t total = (int64_t)a.ntiles_n * a.B * a.H;
+    a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, once);
+    return launch_flat(kern, total, C::NTHREADS, C::LDS_BYTES, stream, a);
 }
 
 } // namespace fb

@@ -316,6 +316,7 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
     };
 
     int it = 0, stg = 0; // stg: the stage of tile `it` (columns); the rows are one stage ahead
+    int turn = __builtin_amdgcn_readfirstlane(cu_slot());
     auto tile = [&](auto edge_tag) {
         constexpr bool EDGE = decltype(edge_tag)::value;
         const int n0 = it * C::BN;
@@ -323,6 +324,7 @@ __device__ __forceinline__ void bwd_dq_lean_body(const BwdArgs &a, int wg, const
         // has used what it read of tile it - 2
         wait_tiles(min(2, ntiles_k - 2 - it));
         asm volatile("s_barrier" ::: "memory");
+        take_turn(turn, a.slots); // (the two workgroups of a compute unit swap wave priority at every tile, as in the forward)
         if (it + C::NSTAGE - 2 < ntiles_k) issue(stg < 2 ? stg + C::NSTAGE - 2 : stg - 2, it + C::NSTAGE - 2);
         if (EDGE) hide(s0, n0);
         FB_SLOT_END;
@@ -378,7 +380,9 @@ static hipError_t launch_dq_lean(const BwdArgs &a0, hipStream_t stream) {
     static KernelOnce once;
     const hipError_t e = allow_lds(kern, C::LDS_BYTES, once);
     if (e != hipSuccess) return e;
-    return launch_flat(kern, (int64_t)a.ntiles_m * a.B * a.H, C::NTHREADS, C::LDS_BYTES, stream, a);
+    const int64_t total = (int64_t)a.ntiles_m * a.B * a.H;
+    a.slots = slots_per_cu(kern, C::NTHREADS, C::LDS_BYTES, total, once);
+    return launch_flat(kern, total, C::NTHREADS, C::LDS_BYTES, stream, a);
 }
 
 } // namespace fb

@@ -481,8 +481,9 @@ __device__ __forceinline__ void store_acc_rows(uint16_t *row, bool row_ok, bool 
 // whenever the older one ends the other is left alone with a SIMD it cannot fill.  Raising the
 // wave priority of a different workgroup at every step evens the progress out.  Measured at
 // B2 H4 d32 r8: forward 5 % faster at L = 8192 and 16384, 4 % at 32768; dq kernel 2 % at 16384;
-// the dk/dv kernel (three workgroups per CU, one 32-query step per turn) gained nothing from any
-// rotation tried and does not take turns.
+// the streamlined dq and dk/dv kernels (two workgroups per CU, a turn per 64-row tile) 0.6 % and 1 %;
+// the general dk/dv kernel (three workgroups per CU, one 32-query step per turn) gained nothing from
+// any rotation tried and does not take turns.
 //
 // cu_slot(): which of the CU's equally sized LDS allocations this workgroup holds (0, 1, ...),
 // read from the LDS_ALLOC hardware register (id 6: base in bits 11:0, size in bits 23:12, same
