@@ -51,6 +51,7 @@ static hipError_t launch_both_lean(const BwdArgs &a0, hipStream_t stream) {
     const hipError_t e = allow_lds(kern, lds, once);
     if (e != hipSuccess) return e;
     const int64_t total = ((int64_t)a.ntiles_m + a.ntiles_n) * a.B * a.H;
+    a.slots = slots_per_cu(kern, 256, lds, total, once);
     return launch_flat(kern, total, 256, lds, stream, a);
 }
 
