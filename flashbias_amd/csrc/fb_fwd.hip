@@ -584,9 +584,11 @@ static hipError_t launch_fwd_cfg(const FwdArgs &a, hipStream_t stream) {
         // On grids that fill the chip a loop of at least 512 keys pays for the kernel's pipeline (4096 x 16
         // windows, general against streamlined: 1.91 against 2.82 ms at 128 keys, 1.79 against 1.88 at 256,
         // 1.38 against 1.21 at 512); small grids take it at every length.
-        if (vec && fwd_lean_ok(a) && (a.Lk >= 512 || small_grid(a.B, a.H, a.Lq)))
+        if (vec && fwd_lean_ok(a) && (a.Lk >= 512 || small_grid(a.B, a.H, a.Lq))) {
+            if (a.causal) return launch_fwd_lean<T, NKR, 1, true>(a, stream);
             return wgs >= num_cus() && !half_empty_256(a.Lq) ? launch_fwd_lean<T, NKR, 2>(a, stream)
                                                              : launch_fwd_lean<T, NKR, 1>(a, stream);
+        }
     }
     if constexpr (NKR <= 2) {
         if (vec && fold_scale_ok<T>(a.scale, a.r, a.Lk)) return launch_fwd_vec<T, NKD, NKR, NDV, true, false, true>(a, stream);

@@ -1,5 +1,6 @@
 // Streamlined forward kernel for the shapes the benchmark family lives on: aligned tensors, no
-// additive or causal mask, head dim 32, rank 8 (or no factors), grids that fill the chip.  Included by
+// additive mask, head dim 32, rank 8 (or no factors); under a causal mask in its instantiation with one
+// query block per wave.  Included by
 // fb_fwd.hip after the general kernel.  What differs from fwd_kernel is the arithmetic per score
 // and the way tiles reach LDS:
 //
@@ -42,11 +43,15 @@ namespace fb {
 // position: all lanes on, one tensor per instruction, nothing but a scalar base and m0 to set up.
 // QB_: query blocks (of 32) per wave.  Two where the grid fills the chip (every key / value fragment
 // read from LDS then feeds two blocks); one on small grids, which doubles the number of waves.
-template <class T, int NKR_, int QB_ = 2>
+// CAUSAL_: the causal instantiation (one query block per wave only: a wave's blocks share one reference point, and
+// under a causal mask the reference point of a query may depend on nothing but the keys that query sees).
+template <class T, int NKR_, int QB_ = 2, bool CAUSAL_ = false>
 struct FwdLeanCfg {
     static constexpr int NKD = 2, NKR = NKR_, NK = NKD + NKR_, QB = QB_;
+    static constexpr bool CAUSAL = CAUSAL_;
     static_assert(NKR_ <= 1, "rank <= 8");
     static_assert(QB_ == 1 || QB_ == 2, "");
+    static_assert(!CAUSAL_ || QB_ == 1, "");
     static constexpr int NWAVES = 4, NTHREADS = 256, BM = 128 * QB_, BN = 128, KB = BN / 32;
     static constexpr int K_BYTES = BN * 64, B_BYTES = NKR_ ? BN * 32 : 0, V_BYTES = BN * 64;
     static constexpr int B_OFF = K_BYTES, V_OFF = K_BYTES + B_BYTES, STAGE_BYTES = V_OFF + V_BYTES;
@@ -79,9 +84,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
     const int c = lane & 31, g = lane >> 5;
 
     const int total = a.ntiles_m * a.B * a.H;
-    const int work = xcd_remap(blockIdx.x, total);
-    const int bh = work / a.ntiles_m;
-    const int tile_m = work % a.ntiles_m;
+    int bh, tile_m;
+    work_order(blockIdx.x, a.ntiles_m, total, C::CAUSAL, bh, tile_m);
+    if (C::CAUSAL) tile_m = a.ntiles_m - 1 - tile_m; // the last query tile sees the most keys
     const int b = bh / a.H, h = bh % a.H;
     const int m0 = tile_m * C::BM;
     const int wq0 = m0 + wave * (32 * QB); // first query of this wave
@@ -109,7 +114,9 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
             qbr[qb][0] = fold_scale_chunk<T>(load_chunk<true>(qbbase, a.qb.ss, query, a.Lq, 0, a.r), kLog2e, true, g == 1);
     }
 
-    const int ntiles_k = (a.Lk + C::BN - 1) / C::BN;
+    // (causal: keys past the workgroup's last query are hidden from all of it)
+    const int k_end = C::CAUSAL ? min(a.Lk, m0 + C::BM) : a.Lk;
+    const int ntiles_k = (k_end + C::BN - 1) / C::BN;
 
     // ---- the copies.  This lane's place in an instruction's 8 lines and what belongs there
     const int dline = lane >> 3, dslot = (lane & 7) ^ ((lane >> 4) & 3);
@@ -192,12 +199,13 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         if constexpr (NKR > 0) acc = T::mfma(f[NKD], qbr[qb][0], acc);
         return acc;
     };
-    // -inf for keys past the end
+    // -inf for keys past the end (causal: and for the keys behind this lane's query)
     auto hide = [&](f32x16_t &s, int ns) {
+        const int last = C::CAUSAL ? min(a.Lk - 1, wq0 + c) : a.Lk - 1;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int key = ns + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (key >= a.Lk) s[v] = -INFINITY;
+            if (key > last) s[v] = -INFINITY;
         }
     };
 
@@ -276,7 +284,7 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
         const int n0 = it * C::BN;
         take_turn(turn, a.slots);
         if (it + 2 < ntiles_k) issue((STG + 2) % 3, n0 + 2 * C::BN);
-        const bool edge = n0 + C::BN > a.Lk;
+        const bool edge = n0 + C::BN > a.Lk || (C::CAUSAL && n0 + C::BN - 1 > wq0); // (the wave's diagonal lies in this tile or before it)
         f32x16_t s_cur, s_nxt;
         read_ka(ka, STG, 0);
         s_cur = scores(ka, 0, minit);
@@ -358,20 +366,23 @@ __global__ __launch_bounds__(C::NTHREADS) __attribute__((amdgpu_waves_per_eu(2, 
 // product: harmless for logits of order one, visible in o for logits in the tens, hence the bound
 // scale * log2(e) <= 1 (which also keeps the folded operand inside the 16-bit range; what a folded
 // factor cannot hold ends up as inf / NaN row sums, which take the fallback).
-// Not for causal calls nor for fewer than 128 keys: with a reference point that is not the row's
-// own maximum the largest P of a row is not exactly 1, so a row that sees one or two keys comes
-// out an ulp off v (the general kernel returns it exactly), and the reference point of a query
-// depends on keys that only the other query of its lane may see, which breaks the bit-for-bit
-// independence of o[i] from keys j > i.
+// Not for fewer than 128 keys.  Under a causal mask only with one query block per wave: the reference
+// point is then the maximum over the keys of the first block that the lane's own query sees, so a row
+// that sees one key has P = 1 and comes out as v exactly, and o[i] does not depend on any key j > i,
+// bit for bit, as with the general kernel.  (With two blocks per wave the two queries of a lane share
+// one reference point, which would make o[i] depend on keys that only query i + 32 sees; a second
+// reference block costs 16 registers the kernel does not have.)  Measured against the general forward,
+// causal: B1 H50 L=8192 r8 0.398 -> 0.337 ms, L=2048 0.039 -> 0.035, B2 H4 L=4096 0.053 -> 0.035,
+// B8 H4 L=16384 without factors 0.85 -> 0.68.
 inline bool fwd_lean_ok(const FwdArgs &a) {
     const int64_t lim = (int64_t)1 << 24; // (32-bit tile row offsets in the copies)
-    return a.d == 32 && (a.r == 8 || a.r == 0) && !a.causal && a.Lk >= 128 && a.scale > 1e-6f && a.scale * kLog2e <= 1.f &&
+    return a.d == 32 && (a.r == 8 || a.r == 0) && a.Lk >= 128 && a.scale > 1e-6f && a.scale * kLog2e <= 1.f &&
            a.k.ss < lim && a.v.ss < lim && (a.r == 0 || a.kb.ss < lim);
 }
 
-template <class T, int NKR, int QB>
+template <class T, int NKR, int QB, bool CAUSAL = false>
 static hipError_t launch_fwd_lean(const FwdArgs &a0, hipStream_t stream) {
-    typedef FwdLeanCfg<T, NKR, QB> C;
+    typedef FwdLeanCfg<T, NKR, QB, CAUSAL> C;
     FwdArgs a = a0;
     a.ntiles_m = (a.Lq + C::BM - 1) / C::BM;
     auto kern = fwd_lean_kernel<T, C>;

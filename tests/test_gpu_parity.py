@@ -274,19 +274,27 @@ def test_lse_and_default_scale(gpu_device):
     assert scale0 == scale and torch.equal(o0, o)  # 0 falls back to the default like `or` does
 
 
-def test_causal_structure_is_exact(gpu_device):
+@pytest.mark.parametrize("B,L,H,d,r", [
+    (2, 333, 3, 32, 8),     # small grid: the streamlined causal forward (one query block per wave)
+    (8, 700, 16, 32, 8),    # the same on a grid that fills the chip, several key tiles
+    (4, 1100, 8, 32, 0),    # ... without factors
+    (2, 333, 3, 32, 16),    # the general forward
+    (2, 400, 2, 64, 8)])
+def test_causal_structure_is_exact(gpu_device, B, L, H, d, r):
     """o[:, 0] == v[:, 0] bit for bit, and changing k / v / k_bias at keys j > i leaves o[i]
     bit-identical (top-left aligned causal mask, flash_bias_triton.py:262)."""
     dev = gpu_device
     q, k, v, qb, kb, _ = [t.to(dev) if t is not None else None
-                          for t in make_inputs(2, 333, 333, 3, 32, 8, torch.bfloat16, seed=4)]
+                          for t in make_inputs(B, L, L, H, d, r, torch.bfloat16, seed=4)]
     o = flash_bias_func(q, k, v, qb, kb, None, True, None)
     assert torch.equal(o[:, 0], v[:, 0])
-    for cut in (1, 64, 65, 200, 332):
-        k2, v2, kb2 = k.clone(), v.clone(), kb.clone()
+    for cut in (1, 64, 65, 200, L - 1):
+        k2, v2 = k.clone(), v.clone()
+        kb2 = kb.clone() if r else None
         k2[:, cut:] += 3
         v2[:, cut:] -= 5
-        kb2[:, cut:] *= -2
+        if r:
+            kb2[:, cut:] *= -2
         o2 = flash_bias_func(q, k2, v2, qb, kb2, None, True, None)
         assert torch.equal(o[:, :cut], o2[:, :cut]), cut
         assert not torch.equal(o[:, cut:], o2[:, cut:]), cut
@@ -940,16 +948,17 @@ def test_random_configurations(gpu_device, B, H, Lq, Lk, d, r, causal, dtype, ma
 @pytest.mark.parametrize("causal", [False, True])
 def test_streamlined_kernels(gpu_device, dtype, r, causal):
     """Head dim 32, rank 8 or no factors, aligned, unmasked, on grids that fill an MI355X: the shapes
-    that take the streamlined forward kernel (not causal, at least two 256-query workgroups per
-    compute unit) and the streamlined dk/dv kernel (at least two 128-key workgroups per compute
+    that take the streamlined forward kernel (two query blocks per wave, at least two 256-query workgroups per
+    compute unit; under a causal mask its one-block instantiation) and the streamlined dk/dv kernel (at least two 128-key workgroups per compute
     unit), with ragged last tiles on both sides, in both element types."""
     B, H, Lq, Lk = (8, 32, 1800, 600) if causal else (8, 16, 1000, 1000)
     assert B * H * ((Lq + 255) // 256) >= 2 * 256 and B * H * ((Lk + 127) // 128) >= 2 * 256
     _case(gpu_device, B, Lq, Lk, H, 32, r, dtype, causal, seed=14)
 
 
+@pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("which", ["q_bias", "k_bias", "logits"])
-def test_streamlined_kernels_fall_back(gpu_device, which):
+def test_streamlined_kernels_fall_back(gpu_device, which, causal):
     """Inputs the streamlined kernels cannot take make their workgroups run the general algorithm
     instead: an fp16 factor entry that overflows once log2(e) is folded into it (60000, facing a zero
     column of the other factor, so the bias itself is unchanged: q_bias for the forward and dq
@@ -966,8 +975,8 @@ def test_streamlined_kernels_fall_back(gpu_device, which):
         zero[..., 3] = 0
         big[:, ::7, :, 3] = 60000.0
         do = (do.float() * 0.03).half()  # (keeps the gradient of the zero column, ~ 60000 dS, inside fp16)
-    ref = oracle(q, k, v, qb, kb, None, False, None, do)
-    got = run_gpu(flash_bias_func, q, k, v, qb, kb, None, False, None, do, gpu_device)
+    ref = oracle(q, k, v, qb, kb, None, causal, None, do)
+    got = run_gpu(flash_bias_func, q, k, v, qb, kb, None, causal, None, do, gpu_device)
     _gate(got, ref, torch.float16)
 
 
